@@ -1,10 +1,10 @@
 """Configuration of hybrid decoders: a stack whose layers each pick one
-sequence mixer (recurrent, state-space, windowed latent attention or
-grouped-query window attention) and one feed-forward (dense, table-routed
-experts, router-chosen experts, or none).
+sequence mixer (recurrent, state-space, gated linear attention, windowed
+latent attention or grouped-query attention) and one feed-forward (dense,
+table-routed experts, router-chosen experts, or none).
 
 The Bizusun design is the first family described this way, Kuforax the
-second.  Everything that
+second, Vurivik the third.  Everything that
 can differ between two models of a family is a field here and is read from
 the checkpoint's ``config.json``; constants that the design fixes (the decay
 constant of the delta rule, its key epsilon) are defaults of the mixer
@@ -28,6 +28,19 @@ class DeltaRuleSpec:
     decay_scale: float = math.exp(-0.5)   # w = exp(-decay_scale * sigmoid(.))
     key_eps: float = 1e-6                 # unit key: k / sqrt(sum k^2 + eps)
     kind: str = "general_delta"
+
+
+@dataclass
+class GLASpec:
+    """Gated linear attention: a matrix state per head with one decay per
+    key channel, ``decay = sigmoid(low-rank projection + bias)^(1/tau)``;
+    the query is scaled by ``dim^(-1/2)``."""
+    heads: int
+    dim: int
+    vdim: int
+    tau: float
+    decay_rank: Optional[int] = None      # rows of a1; None = from the tensor
+    kind: str = "gla"
 
 
 @dataclass
@@ -104,6 +117,9 @@ class RopeSpec:
         return out, self.amp_slope * math.log(self.factor) + 1.0
 
 
+UNBOUNDED = 1 << 30       # a window no sequence reaches
+
+
 @dataclass
 class WindowAttnSpec:
     """Grouped-query softmax attention over a sliding window of a paged
@@ -114,7 +130,11 @@ class WindowAttnSpec:
     sigmoid output gate per head (``head_gate``), and a learned bias per
     (distance bucket, head) added to the scaled scores (``bias_far`` > 0:
     the bucket of distance n is n below half the table's rows, logarithmic
-    steps up to ``bias_far`` above)."""
+    steps up to ``bias_far`` above), biases on the query / key / value
+    projections (``qkv_bias``), one learned logit per head that joins the
+    softmax denominator without a key or a value (``sink``), and a query
+    temperature ``1 + q_temp_coef * ln(floor((p + 1) / q_temp_every) + 1)``
+    at position p.  ``window = UNBOUNDED`` is plain causal attention."""
     heads: int
     kv_heads: int
     dim: int
@@ -122,6 +142,10 @@ class WindowAttnSpec:
     window: int
     scale: float
     keep_first: int = 0
+    qkv_bias: bool = False
+    sink: bool = False
+    q_temp_coef: float = 0.0
+    q_temp_every: int = 1
     rope: Optional[RopeSpec] = None
     qk_norm: bool = False
     values_from_keys: bool = False
@@ -159,6 +183,23 @@ class FFSpec:
     group_keep: int = 1
     shared_ff: int = 0
     weight_eps: float = 1e-20
+    # dense: "silu" is silu(gate) * up; "clamped" is g * sigmoid(slope * g)
+    # * (u + shift) with g = min(gate, limit), u = clamp(up, -limit, limit)
+    act: str = "silu"
+    limit: float = 0.0
+    gate_slope: float = 1.702
+    up_shift: float = 1.0
+    bias: bool = False        # gate / up / down projections carry biases
+
+
+@dataclass
+class BigramSpec:
+    """Hashed pair embedding: row (prev * mul_prev + cur * mul_cur) mod
+    buckets of a (buckets + 1)-row table; a sequence's first token reads
+    the last row."""
+    buckets: int
+    mul_prev: int
+    mul_cur: int
 
 
 @dataclass
@@ -181,12 +222,26 @@ class HybridConfig:
     # "canon": norm -> convolution -> mixer, norm -> ff, token-side input
     # (scalar norm weights).  "sandwich": x += norm(mixer(norm(x))),
     # x += norm(ff(norm(x))) with per-channel weights stored as offsets
-    # from ``norm_offset``.
+    # from ``norm_offset``.  "prenorm": x += m * mixer(norm(x)),
+    # x += m * ff(norm(x)), x += m * token-side input, with per-channel
+    # weights and m = ``residual_mult``.
     layer_style: str = "canon"
     norm_offset: float = 0.0
+    residual_mult: float = 1.0
+    # the embedding: table row * embed_scale [+ hashed pair row]
+    # [+ sinusoid of the position: entry 2i = sin(p * base^(-2i/width)),
+    # entry 2i+1 = cos of the same angle; 0 = none]
+    embed_scale: float = 1.0
+    bigram: Optional[BigramSpec] = None
+    sin_pos_base: float = 0.0
     # layers [start, stop) run ``times`` times in a row with the same
     # weights; every pass owns its cache rows and state
     loop: Optional[tuple] = None
+    # before every pass after the first the embedding output is added to
+    # the stream again (``loop_reinject``); before every pass a learned
+    # vector of that pass is added (``loop_step``, tensor 'loop.step')
+    loop_reinject: bool = False
+    loop_step: bool = False
 
     # the engine's generic accessors
     @property
@@ -205,6 +260,16 @@ class HybridConfig:
             return list(range(n))
         a, b, t = self.loop
         return list(range(a)) + list(range(a, b)) * t + list(range(b, n))
+
+    def pass_starts(self) -> dict:
+        """Run index -> pass number for the first run of every pass of the
+        looped span (empty without a loop)."""
+        if not self.loop:
+            return {}
+        a, b, t = self.loop
+        if b <= a:
+            return {}
+        return {a + r * (b - a): r for r in range(t)}
 
     def cache_owner(self, li: int) -> Optional[int]:
         """Layer whose latent cache layer ``li`` reads (itself unless it
@@ -227,6 +292,8 @@ class HybridConfig:
                 if (src.kv_rank, src.rot_dim) != (m.kv_rank, m.rot_dim):
                     raise ValueError(f"layer {li}: a shared cache needs "
                                      "equal latent and rotated sizes")
+            if m.kind == "gla":
+                assert m.heads > 0 and m.dim > 0 and m.vdim > 0 and m.tau > 0
             if m.kind == "mamba2":
                 assert m.heads % m.groups == 0
                 assert m.inner % m.norm_groups == 0
@@ -237,6 +304,9 @@ class HybridConfig:
                 if m.bias_far > 0 and m.keep_first > 0:
                     raise ValueError(f"layer {li}: the distance bias covers "
                                      "the window only (no kept first tokens)")
+            if L.ff is not None and L.ff.kind == "dense":
+                assert L.ff.act in ("silu", "clamped")
+                assert L.ff.act == "silu" or L.ff.limit > 0
             if L.ff is not None and L.ff.kind == "moe":
                 assert 0 < L.ff.top <= L.ff.experts
             if L.ff is not None and L.ff.kind == "routed_moe":
@@ -245,6 +315,8 @@ class HybridConfig:
                 assert total % f.group_count == 0
                 assert 0 < f.group_keep <= f.group_count
                 assert 0 < f.top <= f.group_keep * (total // f.group_count)
+        if (self.loop_reinject or self.loop_step) and not self.loop:
+            raise ValueError("pass inputs need a looped span")
         if self.loop is not None:
             a, b, t = self.loop
             assert 0 <= a <= b <= len(self.layers) and t >= 1
@@ -516,6 +588,123 @@ def kuforax_preset(width: int, layers: int, vocab: int = 32000,
                         norm_offset=1.0, loop=loop).validate()
 
 
+def _vurivik_mixer_from_json(kind: str, m: dict):
+    """Vurivik mixers: 'gla' (gated linear attention) and 'attention'
+    (causal grouped-query attention with projection biases, a softmax sink
+    and a position-dependent query temperature; no rotation)."""
+    if kind == "gla":
+        return GLASpec(heads=int(m["heads"]), dim=int(m["dim"]),
+                       vdim=int(m["vdim"]), tau=float(m["tau"]))
+    if kind == "attention":
+        qt = m.get("q_temp") or {}
+        return WindowAttnSpec(
+            heads=int(m["heads"]), kv_heads=int(m["kv_heads"]),
+            dim=int(m["dim"]), vdim=int(m["vdim"]), window=UNBOUNDED,
+            scale=float(m["scale"]), qkv_bias=True, sink=True,
+            q_temp_coef=float(qt.get("coef", 0.0)),
+            q_temp_every=int(qt.get("every", 1)))
+    raise ValueError(f"unknown mixer type {kind!r}")
+
+
+def _clamped_ff_from_json(f: Optional[dict]) -> Optional[FFSpec]:
+    if f is None:
+        return None
+    if f["kind"] != "dense":
+        raise ValueError(f"unknown feed-forward kind {f['kind']!r}")
+    return FFSpec(kind="dense", ff=int(f["ff"]), act="clamped",
+                  limit=float(f["limit"]), bias=True)
+
+
+def vurivik_config_from_json(d: dict) -> HybridConfig:
+    """Read a Vurivik ``config.json`` (already parsed)."""
+    layers = [HybridLayerSpec(_vurivik_mixer_from_json(L["type"], L["mixer"]),
+                              _clamped_ff_from_json(L.get("mlp")))
+              for L in d["layers"]]
+    emb = d.get("embedding") or {}
+    bg = emb.get("bigram")
+    loop = d.get("loop")
+    return HybridConfig(
+        arch="vurivik", vocab_size=int(d["vocab"]),
+        hidden_size=int(d["width"]), layers=layers,
+        norm_eps=float(d["norm"]["eps"]), canon_taps=1,
+        token_side_dim=int((d.get("token_side") or {}).get("dim", 0)),
+        layer_style="prenorm",
+        residual_mult=float(d.get("residual_mult", 1.0)),
+        embed_scale=float(emb.get("scale", 1.0)),
+        bigram=None if not bg else BigramSpec(
+            buckets=int(bg["buckets"]), mul_prev=int(bg["mul_prev"]),
+            mul_cur=int(bg["mul_cur"])),
+        sin_pos_base=10000.0,
+        loop=None if not loop else (int(loop["start"]), int(loop["stop"]),
+                                    int(loop["times"])),
+        loop_reinject=bool(loop), loop_step=bool(loop)).validate()
+
+
+def vurivik_config_to_json(cfg: HybridConfig) -> dict:
+    """Inverse of :func:`vurivik_config_from_json` (checkpoint export)."""
+    layers = []
+    for L in cfg.layers:
+        m = L.mixer
+        if m.kind == "gla":
+            mj = {"heads": m.heads, "dim": m.dim, "vdim": m.vdim,
+                  "tau": m.tau}
+        else:
+            mj = {"heads": m.heads, "kv_heads": m.kv_heads, "dim": m.dim,
+                  "vdim": m.vdim, "scale": m.scale,
+                  "q_temp": {"coef": m.q_temp_coef, "every": m.q_temp_every}}
+        fj = None if L.ff is None else \
+            {"kind": "dense", "ff": L.ff.ff, "limit": L.ff.limit}
+        layers.append({"type": m.kind, "mixer": mj, "mlp": fj})
+    emb = {"scale": cfg.embed_scale}
+    if cfg.bigram is not None:
+        emb["bigram"] = {"buckets": cfg.bigram.buckets,
+                         "mul_prev": cfg.bigram.mul_prev,
+                         "mul_cur": cfg.bigram.mul_cur}
+    out = {"architecture": "Vurivik", "vocab": cfg.vocab_size,
+           "width": cfg.hidden_size, "embedding": emb, "layers": layers,
+           "norm": {"eps": cfg.norm_eps},
+           "residual_mult": cfg.residual_mult,
+           "token_side": {"dim": cfg.token_side_dim}}
+    if cfg.loop is not None:
+        out["loop"] = {"start": cfg.loop[0], "stop": cfg.loop[1],
+                       "times": cfg.loop[2]}
+    return out
+
+
+def vurivik_preset(width: int, layers: int, vocab: int = 32000,
+                   heads: int = 16, kv_heads: int = 4, ff_mult: float = 2.75,
+                   gla_every: int = 3, gla_heads: int = 0,
+                   loop: Optional[tuple] = None) -> HybridConfig:
+    """A Vurivik stack of realistic layer sizes (random weights): every
+    ``gla_every``-th layer is gated linear attention without a feed-forward,
+    the others causal grouped-query attention with the clamped gated
+    feed-forward."""
+    hd = width // heads
+    gh = gla_heads or max(1, heads // 2)
+    out = []
+    for li in range(layers):
+        if gla_every and li % gla_every == gla_every - 1:
+            out.append(HybridLayerSpec(
+                GLASpec(heads=gh, dim=hd, vdim=2 * hd, tau=16.0,
+                        decay_rank=16), None))
+        else:
+            out.append(HybridLayerSpec(
+                WindowAttnSpec(heads=heads, kv_heads=kv_heads, dim=hd,
+                               vdim=hd, window=UNBOUNDED,
+                               scale=1.0 / math.sqrt(hd), qkv_bias=True,
+                               sink=True, q_temp_coef=0.1, q_temp_every=1024),
+                FFSpec(kind="dense", ff=int(width * ff_mult) // 64 * 64,
+                       act="clamped", limit=7.0, bias=True)))
+    return HybridConfig(
+        arch="vurivik", vocab_size=vocab, hidden_size=width, layers=out,
+        norm_eps=1e-5, canon_taps=1, token_side_dim=max(8, width // 16),
+        layer_style="prenorm", residual_mult=0.5,
+        embed_scale=math.sqrt(width),
+        bigram=BigramSpec(buckets=65521, mul_prev=31, mul_cur=7),
+        sin_pos_base=10000.0, loop=loop, loop_reinject=bool(loop),
+        loop_step=bool(loop)).validate()
+
+
 def read_config_dir(path: str):
     """Model config from a checkpoint folder's ``config.json``.  The
     ``architecture`` key names the family; HF-style folders
@@ -527,6 +716,8 @@ def read_config_dir(path: str):
         return bizusun_config_from_json(d)
     if arch == "Kuforax":
         return kuforax_config_from_json(d)
+    if arch == "Vurivik":
+        return vurivik_config_from_json(d)
     mt = d.get("model_type")
     if mt in ("llama", "qwen2"):
         from .registry import DecoderConfig

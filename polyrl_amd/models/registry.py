@@ -107,8 +107,22 @@ MODEL_CONFIGS = {
 
 
 def _hybrid_presets():
-    from .hybrid import bizusun_preset, kuforax_preset
+    from .hybrid import bizusun_preset, kuforax_preset, vurivik_preset
     return {
+        # tiny looped stack for CPU unit tests / fast GPU smoke
+        "vurivik-debug": lambda: vurivik_preset(
+            width=64, layers=4, vocab=300, heads=4, kv_heads=2, ff_mult=2.5,
+            gla_every=2, gla_heads=2, loop=(1, 3, 2)),
+        # bench pairs: beside llama-400m / llama3-1b / llama3-8b-l8
+        "vurivik-400m": lambda: vurivik_preset(
+            width=1024, layers=12, vocab=32000, heads=16, kv_heads=4,
+            ff_mult=4.0, gla_every=3),
+        "vurivik-1b": lambda: vurivik_preset(
+            width=2048, layers=16, vocab=128256, heads=32, kv_heads=8,
+            ff_mult=4.0, gla_every=4),
+        "vurivik-8b-l8": lambda: vurivik_preset(
+            width=4096, layers=8, vocab=128256, heads=32, kv_heads=8,
+            ff_mult=3.5, gla_every=4),
         # tiny looped stack for CPU unit tests / fast GPU smoke
         "kuforax-debug": lambda: kuforax_preset(
             width=64, layers=3, vocab=300, heads=4, kv_heads=2, experts=6,

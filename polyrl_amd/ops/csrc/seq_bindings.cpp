@@ -5,14 +5,24 @@
 
 void seq_add_rmsnorm(torch::Tensor out, torch::Tensor res, torch::Tensor y,
                      torch::Tensor weight, double eps, int64_t mode,
-                     double offset, torch::Tensor weight2);
+                     double offset, torch::Tensor weight2, double y_scale,
+                     torch::Tensor extra, torch::Tensor extra_vec);
+void seq_embed_compose(torch::Tensor out, torch::Tensor table,
+                       torch::Tensor tokens, double scale,
+                       torch::Tensor pair_table, torch::Tensor prev_tokens,
+                       int64_t mul_prev, int64_t mul_cur, int64_t buckets,
+                       torch::Tensor positions, torch::Tensor inv_freq);
+void seq_gla_scan(torch::Tensor out, torch::Tensor q, torch::Tensor k,
+                  torch::Tensor v, torch::Tensor z_lin, torch::Tensor z_bias,
+                  torch::Tensor state, torch::Tensor cu_q,
+                  torch::Tensor state_slot, double q_scale, double inv_tau);
 void seq_causal_conv(torch::Tensor out, torch::Tensor x, torch::Tensor w,
                      torch::Tensor bias, torch::Tensor state,
                      torch::Tensor cu_q, torch::Tensor state_slot,
                      torch::Tensor seq_of_tok, bool add_input, bool act_silu);
 void seq_group_rmsnorm(torch::Tensor out, torch::Tensor y,
                        torch::Tensor weight, int64_t groups, double eps,
-                       torch::Tensor gate);
+                       torch::Tensor gate, int64_t gate_act);
 void seq_rope_partial(torch::Tensor q, int64_t offset, torch::Tensor inv_freq,
                       torch::Tensor positions);
 void seq_latent_kv_store(torch::Tensor dkv, int64_t rank, torch::Tensor norm_w,
@@ -20,7 +30,7 @@ void seq_latent_kv_store(torch::Tensor dkv, int64_t rank, torch::Tensor norm_w,
                          torch::Tensor inv_freq, torch::Tensor cache,
                          torch::Tensor slot_mapping);
 void seq_act_mul(torch::Tensor out, torch::Tensor a, torch::Tensor b,
-                 int64_t mode);
+                 int64_t mode, double p0, double p1, double p2);
 void seq_gelu_mul_rows(torch::Tensor out, torch::Tensor gate,
                        torch::Tensor table, torch::Tensor tokens,
                        int64_t col0);
@@ -67,14 +77,16 @@ void seq_gqa_window_attention(torch::Tensor out, torch::Tensor q,
                               int64_t D, int64_t Dv, int64_t window,
                               int64_t keep_first, torch::Tensor rel,
                               torch::Tensor dist_bucket, torch::Tensor gate,
-                              double scale);
+                              double scale, torch::Tensor sink,
+                              double q_temp_coef, int64_t q_temp_every);
 void seq_gqa_window_attention_mfma(
     torch::Tensor out, torch::Tensor q, torch::Tensor tile_n0,
     torch::Tensor tile_cnt, torch::Tensor cache, torch::Tensor page_table,
     torch::Tensor seq_of_tok, torch::Tensor positions, int64_t H, int64_t G,
     int64_t D, int64_t Dv, int64_t window, int64_t keep_first,
     torch::Tensor rel, torch::Tensor dist_bucket, torch::Tensor gate,
-    double scale);
+    double scale, torch::Tensor sink, double q_temp_coef,
+    int64_t q_temp_every);
 void seq_moe_route(torch::Tensor idx, torch::Tensor w, torch::Tensor logits,
                    torch::Tensor correction, int64_t groups, int64_t keep);
 void seq_moe_routed_ffn(torch::Tensor y, torch::Tensor act, torch::Tensor h,
@@ -98,17 +110,21 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "router-chosen plain experts for decode-sized bf16 batches");
   m.def("seq_moe_weighted_combine", &seq_moe_weighted_combine,
         "weighted sum of chosen experts, identity experts and shared");
+  m.def("seq_embed_compose", &seq_embed_compose,
+        "scaled embedding row + hashed pair row + sinusoid, fp32");
+  m.def("seq_gla_scan", &seq_gla_scan,
+        "gated linear attention scan (fp32 state, in place)");
   m.def("seq_add_rmsnorm", &seq_add_rmsnorm,
         "fp32 residual add + RMS norm / cast / unit-RMS add");
   m.def("seq_causal_conv", &seq_causal_conv,
         "stateful depthwise causal convolution over packed rows");
   m.def("seq_group_rmsnorm", &seq_group_rmsnorm,
-        "grouped RMS norm with optional sigmoid gate");
+        "grouped RMS norm with optional sigmoid / SiLU gate");
   m.def("seq_rope_partial", &seq_rope_partial,
         "rotate-half RoPE on a slice of each head, in place");
   m.def("seq_latent_kv_store", &seq_latent_kv_store,
         "norm + rotate + write latent cache rows");
-  m.def("seq_act_mul", &seq_act_mul, "silu*b / sigmoid*b / tanh");
+  m.def("seq_act_mul", &seq_act_mul, "silu*b / sigmoid*b / tanh / gelu / clamped gated unit");
   m.def("seq_gelu_mul_rows", &seq_gelu_mul_rows,
         "gelu_tanh(gate) * table rows gathered by token");
   m.def("seq_moe_combine", &seq_moe_combine,

@@ -16,7 +16,11 @@
 // position p sees key j <= p when p - j < window or j < keep; the two key
 // ranges [0, min(keep, lo)) and [lo, p] are walked as one list.  Scores, the
 // optional distance-bucket bias rel[bucket[p-j], head], the online softmax
-// and the per-head sigmoid gate are fp32.
+// and the per-head sigmoid gate are fp32.  Two further options: a sink, one
+// learned logit per head that joins the softmax denominator once without a
+// key or a value (the running maximum starts at the sink, the running sum at
+// one), and a query temperature that multiplies the score scale of the row at
+// position p by 1 + coef * ln(floor((p + 1) / every) + 1).
 #include <torch/extension.h>
 #include <ATen/hip/HIPContext.h>
 
@@ -212,7 +216,8 @@ __global__ __launch_bounds__(256) void gqa_attn_kernel(
     const int* __restrict__ dist_bucket,   // (window,) or null
     const T* __restrict__ gate, long ldg,  // (N, H) view or null
     int H, int G, int D, int Dv, int page_size, int window, int keep,
-    float scale, bool vec, int lpr) {
+    float scale, bool vec, int lpr, const float* __restrict__ sink,
+    float qt_coef, int qt_every) {
   constexpr int EPL = Vec16<T>::N;
   __shared__ float q_sh[4][NCH * 64];
   __shared__ float p_sh[4][64];
@@ -227,6 +232,8 @@ __global__ __launch_bounds__(256) void gqa_attn_kernel(
   const int pos = positions[n];
   const int b = seq_of_tok[n];
   const int* ptab = page_table + (long)b * max_pages;
+  if (qt_coef != 0.f)
+    scale *= 1.f + qt_coef * logf((float)((pos + 1) / qt_every + 1));
   const int lo = pos - window + 1 > 0 ? pos - window + 1 : 0;
   const int nkeep = keep < lo ? keep : lo;
   const int total = nkeep + (pos - lo + 1);
@@ -240,7 +247,7 @@ __global__ __launch_bounds__(256) void gqa_attn_kernel(
   for (int c = 0; c < NCH; ++c) o[c] = 0.f;
 #pragma unroll
   for (int k = 0; k < EPL; ++k) ov[k] = 0.f;
-  float m = -INFINITY, l = 0.f;
+  float m = sink ? sink[h] : -INFINITY, l = sink ? 1.f : 0.f;
   const int kgrp = lpr ? lane / lpr : 0;          // key of an iteration
   const int dcol = lpr ? (lane % lpr) * EPL : 0;  // first value entry
   const int kper = lpr ? 64 / lpr : 1;            // keys per iteration
@@ -319,7 +326,8 @@ void gqa_attention_check(torch::Tensor out, torch::Tensor q,
                          int64_t H, int64_t G, int64_t D, int64_t Dv,
                          int64_t window, int64_t keep_first,
                          torch::Tensor rel, torch::Tensor dist_bucket,
-                         torch::Tensor gate) {
+                         torch::Tensor gate, torch::Tensor sink,
+                         int64_t q_temp_every) {
   CHECK_I32(page_table); CHECK_I32(seq_of_tok); CHECK_I32(positions);
   const long N = q.size(0);
   TORCH_CHECK(H > 0 && G > 0 && H % G == 0 && D > 0 && Dv > 0 && window >= 1 &&
@@ -347,6 +355,11 @@ void gqa_attention_check(torch::Tensor out, torch::Tensor q,
     TORCH_CHECK(gate.size(0) == N && gate.size(1) == H &&
                 gate.scalar_type() == ty);
   }
+  if (sink.defined() && sink.numel() > 0) {
+    CHECK_F32(sink);
+    TORCH_CHECK(sink.numel() == H, "one sink per query head");
+  }
+  TORCH_CHECK(q_temp_every >= 1, "query temperature period");
 }
 
 #define GQA_LAUNCH(NCHV)                                                      \
@@ -359,7 +372,8 @@ void gqa_attention_check(torch::Tensor out, torch::Tensor q,
       has_gate ? (const T*)gate.data_ptr() : nullptr,                         \
       has_gate ? gate.stride(0) : 0, (int)H, (int)G, (int)D, (int)Dv,         \
       (int)cache.size(1), (int)window, (int)keep_first, (float)scale, vec,     \
-      lpr)
+      lpr, has_sink ? sink.data_ptr<float>() : nullptr, (float)q_temp_coef,   \
+      (int)q_temp_every)
 
 void seq_gqa_window_attention(torch::Tensor out, torch::Tensor q,
                               torch::Tensor cache, torch::Tensor page_table,
@@ -368,11 +382,14 @@ void seq_gqa_window_attention(torch::Tensor out, torch::Tensor q,
                               int64_t D, int64_t Dv, int64_t window,
                               int64_t keep_first, torch::Tensor rel,
                               torch::Tensor dist_bucket, torch::Tensor gate,
-                              double scale) {
+                              double scale, torch::Tensor sink,
+                              double q_temp_coef, int64_t q_temp_every) {
   gqa_attention_check(out, q, cache, page_table, seq_of_tok, positions, H, G,
-                      D, Dv, window, keep_first, rel, dist_bucket, gate);
+                      D, Dv, window, keep_first, rel, dist_bucket, gate, sink,
+                      q_temp_every);
   const int N = q.size(0);
   if (N == 0) return;
+  const bool has_sink = sink.defined() && sink.numel() > 0;
   const bool has_rel = rel.defined() && rel.numel() > 0;
   const bool has_gate = gate.defined() && gate.numel() > 0;
   const int nch = (int)((std::max(D, Dv) + 63) / 64);

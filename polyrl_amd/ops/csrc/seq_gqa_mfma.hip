@@ -11,8 +11,11 @@
 // come from the paged cache rows ([G*D keys | G*Dv values]) into LDS; QK^T
 // and P.V run on v_mfma_f32_16x16x32_bf16 with fp32 accumulators; scale, the
 // optional distance-bucket bias (this head's column of the table sits in
-// LDS), the online softmax and the sigmoid head gate are fp32.  The next
-// tiles are fetched into registers while the current ones are multiplied.
+// LDS), the online softmax and the sigmoid head gate are fp32; so are the
+// optional sink (the running maximum starts at the head's sink, the running
+// sum at one) and the per-row query temperature folded into the score scale.
+// The next tiles are fetched into registers while the current ones are
+// multiplied.
 // K-tile bytes are XOR-swizzled by row inside each 64-byte chunk.
 #include <torch/extension.h>
 #include <ATen/hip/HIPContext.h>
@@ -42,7 +45,8 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(
     const float* __restrict__ rel, int rel_rows,
     const int* __restrict__ dist_bucket,
     const bf16_t* __restrict__ gate, long ldg, int H, int G, int D, int Dv,
-    int page_size, int window, int keep, float scale) {
+    int page_size, int window, int keep, float scale,
+    const float* __restrict__ sink, float qt_coef, int qt_every) {
   constexpr int DKP = KS * 32;           // padded head size in LDS
   constexpr int NVT = KS * 2;            // 16-wide output tiles
   __shared__ __attribute__((aligned(16))) bf16_t Ks[GKV * DKP];
@@ -85,17 +89,20 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(
                         : __builtin_bit_cast(bf16x8_t, zi);
     }
   }
-  float m_run[4], l_run[4];
+  float m_run[4], l_run[4], rscale[4];
   int rpos[4];
   bool rok[4];
   f32x4_t o_acc[NVT];
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const int i = wid * 16 + lhi * 4 + r;
-    m_run[r] = -1e30f;
-    l_run[r] = 0.f;
+    m_run[r] = sink ? sink[h] : -1e30f;
+    l_run[r] = sink ? 1.f : 0.f;
     rpos[r] = pos0 + i;
     rok[r] = i < cnt;
+    rscale[r] = scale;
+    if (qt_coef != 0.f)
+      rscale[r] *= 1.f + qt_coef * logf((float)((rpos[r] + 1) / qt_every + 1));
   }
 #pragma unroll
   for (int nt = 0; nt < NVT; ++nt) o_acc[nt] = {0.f, 0.f, 0.f, 0.f};
@@ -172,7 +179,7 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(
         const int dist = rpos[r] - j;
         const bool live = rok[r] && j <= jmax && dist >= 0 &&
                           (dist < window || j < keep);
-        float sv = c[nt][r] * scale;
+        float sv = c[nt][r] * rscale[r];
         if (rel && live) sv += rel_s[dist_bucket[dist]];
         s[nt] = live ? sv : -1e30f;
       }
@@ -248,7 +255,8 @@ void gqa_attention_check(torch::Tensor out, torch::Tensor q,
                          int64_t H, int64_t G, int64_t D, int64_t Dv,
                          int64_t window, int64_t keep_first,
                          torch::Tensor rel, torch::Tensor dist_bucket,
-                         torch::Tensor gate);
+                         torch::Tensor gate, torch::Tensor sink,
+                         int64_t q_temp_every);
 void seq_gqa_window_attention(torch::Tensor out, torch::Tensor q,
                               torch::Tensor cache, torch::Tensor page_table,
                               torch::Tensor seq_of_tok,
@@ -256,7 +264,8 @@ void seq_gqa_window_attention(torch::Tensor out, torch::Tensor q,
                               int64_t D, int64_t Dv, int64_t window,
                               int64_t keep_first, torch::Tensor rel,
                               torch::Tensor dist_bucket, torch::Tensor gate,
-                              double scale);
+                              double scale, torch::Tensor sink,
+                              double q_temp_coef, int64_t q_temp_every);
 
 #define GQA_MFMA_LAUNCH(KSV)                                                  \
   hipLaunchKernelGGL((gqa_attn_mfma_kernel<KSV>), grid, dim3(256), 0, stream, \
@@ -269,7 +278,9 @@ void seq_gqa_window_attention(torch::Tensor out, torch::Tensor q,
       has_rel ? dist_bucket.data_ptr<int>() : nullptr,                        \
       has_gate ? (const bf16_t*)gate.data_ptr() : nullptr,                    \
       has_gate ? gate.stride(0) : 0, (int)H, (int)G, (int)D, (int)Dv,         \
-      (int)cache.size(1), (int)window, (int)keep_first, (float)scale)
+      (int)cache.size(1), (int)window, (int)keep_first, (float)scale,         \
+      has_sink ? sink.data_ptr<float>() : nullptr, (float)q_temp_coef,        \
+      (int)q_temp_every)
 
 void seq_gqa_window_attention_mfma(
     torch::Tensor out, torch::Tensor q, torch::Tensor tile_n0,
@@ -277,9 +288,12 @@ void seq_gqa_window_attention_mfma(
     torch::Tensor seq_of_tok, torch::Tensor positions, int64_t H, int64_t G,
     int64_t D, int64_t Dv, int64_t window, int64_t keep_first,
     torch::Tensor rel, torch::Tensor dist_bucket, torch::Tensor gate,
-    double scale) {
+    double scale, torch::Tensor sink, double q_temp_coef,
+    int64_t q_temp_every) {
   gqa_attention_check(out, q, cache, page_table, seq_of_tok, positions, H, G,
-                      D, Dv, window, keep_first, rel, dist_bucket, gate);
+                      D, Dv, window, keep_first, rel, dist_bucket, gate, sink,
+                      q_temp_every);
+  const bool has_sink = sink.defined() && sink.numel() > 0;
   CHECK_I32(tile_n0); CHECK_I32(tile_cnt);
   TORCH_CHECK(tile_n0.numel() == tile_cnt.numel());
   const bool has_rel = rel.defined() && rel.numel() > 0;
@@ -289,7 +303,8 @@ void seq_gqa_window_attention_mfma(
       (has_rel && rel.size(0) > GQA_MAX_REL)) {
     seq_gqa_window_attention(out, q, cache, page_table, seq_of_tok, positions,
                              H, G, D, Dv, window, keep_first, rel,
-                             dist_bucket, gate, scale);
+                             dist_bucket, gate, scale, sink, q_temp_coef,
+                             q_temp_every);
     return;
   }
   const int ntiles = tile_n0.numel();

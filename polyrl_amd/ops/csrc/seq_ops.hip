@@ -1,6 +1,7 @@
 // Row-wise kernels of the hybrid decoders: fp32-residual add + RMS norms,
-// stateful depthwise causal convolution, grouped RMS norm with an optional
-// sigmoid gate, partial rotary embedding, the latent-cache writer, gated
+// the composed embedding (scaled row + hashed pair row + sinusoid), stateful
+// depthwise causal convolution, grouped RMS norm with an optional sigmoid or
+// SiLU gate, partial rotary embedding, the latent-cache writer, gated
 // activations, and the expert-output combine.
 //
 // Activations are T (bf16 or fp32); the residual stream, norm statistics,
@@ -15,17 +16,20 @@
 // ------------------------------------------------- residual add + RMS norm
 // g[i] = off + w[i] (w holds 1 or D numbers; off = 0 for plain weights, 1 for
 // weights stored around zero)
-// mode 0: res += y; out = res * rsqrt(mean(res^2)+eps) * g      (norm)
-// mode 1: res += y; out = res (cast)                             (no norm)
-// mode 2: res += y * rsqrt(mean(y^2)+eps) * g                    (out unused)
+// mode 0: res += ys*y [+ ex] [+ exv]; out = res * rsqrt(mean(res^2)+eps) * g
+// mode 1: res += ys*y; out = res (cast)                          (no norm)
+// mode 2: res += ys * y * rsqrt(mean(y^2)+eps) * g               (out unused)
 // mode 3: mode 2, then out = res * rsqrt(mean(res^2)+eps) * (off + w2)
 //         (the joint between two normed sublayers in one pass)
+// ys scales the branch that joins the stream; ex (rows, D) fp32 and exv (D)
+// fp32 are what a pass of a looped span adds at its start.
 template <typename T>
 __global__ __launch_bounds__(256) void add_rmsnorm_kernel(
     T* __restrict__ out, float* __restrict__ res, const T* __restrict__ y,
     long ldy, const float* __restrict__ w, int wn, int D, float eps,
     int mode, bool out_is_res, float off, const float* __restrict__ w2,
-    int w2n) {
+    int w2n, float ys, const float* __restrict__ ex,
+    const float* __restrict__ exv) {
   __shared__ float red[8], red2[8];
   const long row = blockIdx.x;
   float* rr = res + row * D;
@@ -37,12 +41,13 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(
       ss += f * f;
     }
   } else {
+    const float* er = ex ? ex + row * D : nullptr;
     for (int i = threadIdx.x; i < D; i += 256) {
       float f = rr[i];
-      if (yr) {
-        f += ldf(yr + i);
-        rr[i] = f;
-      }
+      if (yr) f += ys * ldf(yr + i);
+      if (er) f += er[i];
+      if (exv) f += exv[i];
+      if (yr || er || exv) rr[i] = f;
       ss += f * f;
     }
   }
@@ -61,7 +66,8 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(
   }
   float ss2 = 0.f;
   for (int i = threadIdx.x; i < D; i += 256) {
-    const float f = rr[i] + ldf(yr + i) * inv * (w[wn == 1 ? 0 : i] + off);
+    const float f =
+        rr[i] + ys * (ldf(yr + i) * inv * (w[wn == 1 ? 0 : i] + off));
     rr[i] = f;
     ss2 += f * f;
   }
@@ -74,7 +80,8 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(
 
 void seq_add_rmsnorm(torch::Tensor out, torch::Tensor res, torch::Tensor y,
                      torch::Tensor weight, double eps, int64_t mode,
-                     double offset, torch::Tensor weight2) {
+                     double offset, torch::Tensor weight2, double y_scale,
+                     torch::Tensor extra, torch::Tensor extra_vec) {
   CHECK_F32(res);
   TORCH_CHECK(res.dim() == 2);
   const int D = res.size(1);
@@ -102,6 +109,18 @@ void seq_add_rmsnorm(torch::Tensor out, torch::Tensor res, torch::Tensor y,
     TORCH_CHECK(w2n == 1 || w2n == D, "norm weight must hold 1 or D numbers");
     w2 = weight2.data_ptr<float>();
   }
+  const float* ex = nullptr;
+  const float* exv = nullptr;
+  if (extra.defined() && extra.numel() > 0) {
+    CHECK_F32(extra);
+    TORCH_CHECK(mode == 0 && extra.numel() == res.numel(), "extra shape");
+    ex = extra.data_ptr<float>();
+  }
+  if (extra_vec.defined() && extra_vec.numel() > 0) {
+    CHECK_F32(extra_vec);
+    TORCH_CHECK(mode == 0 && extra_vec.numel() == D, "extra_vec shape");
+    exv = extra_vec.data_ptr<float>();
+  }
   const bool out_is_res = out.data_ptr() == res.data_ptr();
   TORCH_CHECK(mode != 3 || !out_is_res);
   if (mode != 2) {
@@ -118,7 +137,82 @@ void seq_add_rmsnorm(torch::Tensor out, torch::Tensor res, torch::Tensor y,
       mode == 2 || out_is_res ? nullptr : (T*)out.data_ptr(),
       res.data_ptr<float>(), has_y ? (const T*)y.data_ptr() : nullptr,
       has_y ? y.stride(0) : 0, w, wn, D, (float)eps, (int)mode, out_is_res,
-      (float)offset, w2, w2n); });
+      (float)offset, w2, w2n, (float)y_scale, ex, exv); });
+  HIP_CHECK_KERNEL();
+}
+
+// ------------------------------------------------------ composed embedding
+// out[n] = table[tok] * scale [+ pair[row]] [+ sinusoid(pos)], fp32.
+// row = (prev * mul_prev + tok * mul_cur) mod buckets, or ``buckets`` (the
+// table's last row) where prev < 0.  Sinusoid: entry 2i = sin(a), entry
+// 2i+1 = cos(a), a = fp32(pos) * inv_freq[i].
+template <typename T>
+__global__ __launch_bounds__(256) void embed_compose_kernel(
+    float* __restrict__ out, const T* __restrict__ table,
+    const long* __restrict__ tokens, float scale, const T* __restrict__ pair,
+    const long* __restrict__ prev, long mul_prev, long mul_cur, long buckets,
+    const int* __restrict__ pos, const float* __restrict__ inv_freq, int D) {
+  const long n = blockIdx.x;
+  const long tok = tokens[n];
+  const T* er = table + tok * D;
+  const T* pr = nullptr;
+  if (pair) {
+    const long pv = prev[n];
+    const long row = pv < 0 ? buckets : (pv * mul_prev + tok * mul_cur) % buckets;
+    pr = pair + row * D;
+  }
+  const float p = inv_freq ? (float)pos[n] : 0.f;
+  for (int i = threadIdx.x; i < D; i += 256) {
+    float f = ldf(er + i) * scale;
+    if (pr) f += ldf(pr + i);
+    if (inv_freq) {
+      const float ang = p * inv_freq[i >> 1];
+      f += (i & 1) ? cosf(ang) : sinf(ang);
+    }
+    out[n * D + i] = f;
+  }
+}
+
+void seq_embed_compose(torch::Tensor out, torch::Tensor table,
+                       torch::Tensor tokens, double scale,
+                       torch::Tensor pair_table, torch::Tensor prev_tokens,
+                       int64_t mul_prev, int64_t mul_cur, int64_t buckets,
+                       torch::Tensor positions, torch::Tensor inv_freq) {
+  CHECK_F32(out);
+  TORCH_CHECK(table.is_cuda() && table.is_contiguous() && table.dim() == 2);
+  TORCH_CHECK(tokens.is_cuda() && tokens.dtype() == torch::kInt64 &&
+              tokens.is_contiguous());
+  const long N = tokens.numel();
+  const int D = table.size(1);
+  TORCH_CHECK(out.dim() == 2 && out.size(0) == N && out.size(1) == D);
+  const bool has_pair = pair_table.defined() && pair_table.numel() > 0;
+  if (has_pair) {
+    TORCH_CHECK(pair_table.is_cuda() && pair_table.is_contiguous() &&
+                pair_table.dim() == 2 && pair_table.size(1) == D &&
+                pair_table.scalar_type() == table.scalar_type());
+    TORCH_CHECK(buckets > 0 && pair_table.size(0) == buckets + 1,
+                "the pair table holds buckets + 1 rows");
+    TORCH_CHECK(mul_prev >= 0 && mul_cur >= 0);
+    TORCH_CHECK(prev_tokens.is_cuda() && prev_tokens.dtype() == torch::kInt64 &&
+                prev_tokens.is_contiguous() && prev_tokens.numel() == N);
+  }
+  const bool has_pos = inv_freq.defined() && inv_freq.numel() > 0;
+  if (has_pos) {
+    CHECK_F32(inv_freq);
+    CHECK_I32(positions);
+    TORCH_CHECK(inv_freq.numel() == (D + 1) / 2 && positions.numel() == N);
+  }
+  if (N == 0) return;
+  auto stream = at::hip::getCurrentHIPStream();
+  SEQ_DISPATCH_T(table.scalar_type(), {
+    hipLaunchKernelGGL((embed_compose_kernel<T>), dim3(N), dim3(256), 0,
+        stream, out.data_ptr<float>(), (const T*)table.data_ptr(),
+        (const long*)tokens.data_ptr<int64_t>(), (float)scale,
+        has_pair ? (const T*)pair_table.data_ptr() : nullptr,
+        has_pair ? (const long*)prev_tokens.data_ptr<int64_t>() : nullptr,
+        (long)mul_prev, (long)mul_cur, (long)buckets,
+        has_pos ? positions.data_ptr<int>() : nullptr,
+        has_pos ? inv_freq.data_ptr<float>() : nullptr, D); });
   HIP_CHECK_KERNEL();
 }
 
@@ -216,14 +310,15 @@ void seq_causal_conv(torch::Tensor out, torch::Tensor x, torch::Tensor w,
 }
 
 // ------------------------------------------------ grouped RMS norm (+gate)
-// out = y / rms_group(y) * w * (gate ? sigmoid(gate) : 1).  Small groups
+// out = y / rms_group(y) * w * (gate ? sigmoid(gate) or silu(gate) : 1); w
+// holds D numbers or one group's worth shared by all groups.  Small groups
 // (heads): one wave per (row, group), grid.y covers the groups four at a
 // time.  Large groups (BLOCK): the whole block reduces one (row, group).
 template <typename T, bool BLOCK>
 __global__ __launch_bounds__(256) void group_rmsnorm_kernel(
     T* __restrict__ out, const float* __restrict__ y,
     const float* __restrict__ w, const T* __restrict__ gate, long ldg, int D,
-    int groups, float eps) {
+    int groups, float eps, bool w_shared, int gate_act) {
   __shared__ float red[8];
   const long row = blockIdx.x;
   const int lane = threadIdx.x & 63;
@@ -240,20 +335,26 @@ __global__ __launch_bounds__(256) void group_rmsnorm_kernel(
   const float inv = rsqrtf(ss / gs + eps);
   for (int i = t0; i < gs; i += step) {
     const int c = g * gs + i;
-    float v = yr[i] * inv * w[c];
-    if (gate) v *= sigmoidf_acc(ldf(gate + row * ldg + c));
+    float v = yr[i] * inv * w[w_shared ? i : c];
+    if (gate) {
+      const float gv = ldf(gate + row * ldg + c);
+      v *= gate_act == 2 ? siluf_acc(gv) : sigmoidf_acc(gv);
+    }
     stf(out + row * D + c, v);
   }
 }
 
 void seq_group_rmsnorm(torch::Tensor out, torch::Tensor y,
                        torch::Tensor weight, int64_t groups, double eps,
-                       torch::Tensor gate) {
+                       torch::Tensor gate, int64_t gate_act) {
   CHECK_F32(y);
   CHECK_F32(weight);
   TORCH_CHECK(y.dim() == 2 && out.is_contiguous() && out.sizes() == y.sizes());
   const int D = y.size(1);
-  TORCH_CHECK(groups >= 1 && D % groups == 0 && weight.numel() == D);
+  TORCH_CHECK(groups >= 1 && D % groups == 0 &&
+              (weight.numel() == D || weight.numel() == D / groups));
+  TORCH_CHECK(gate_act == 1 || gate_act == 2);
+  const bool w_shared = weight.numel() != D;
   const bool has_g = gate.defined() && gate.numel() > 0;
   if (has_g) {
     CHECK_ROWS(gate);
@@ -270,13 +371,15 @@ void seq_group_rmsnorm(torch::Tensor out, torch::Tensor y,
           stream, (T*)out.data_ptr(), y.data_ptr<float>(),
           weight.data_ptr<float>(),
           has_g ? (const T*)gate.data_ptr() : nullptr,
-          has_g ? gate.stride(0) : 0, D, (int)groups, (float)eps);
+          has_g ? gate.stride(0) : 0, D, (int)groups, (float)eps, w_shared,
+          (int)gate_act);
     else
       hipLaunchKernelGGL((group_rmsnorm_kernel<T, false>), grid, dim3(256), 0,
           stream, (T*)out.data_ptr(), y.data_ptr<float>(),
           weight.data_ptr<float>(),
           has_g ? (const T*)gate.data_ptr() : nullptr,
-          has_g ? gate.stride(0) : 0, D, (int)groups, (float)eps);
+          has_g ? gate.stride(0) : 0, D, (int)groups, (float)eps, w_shared,
+          (int)gate_act);
   });
   HIP_CHECK_KERNEL();
 }
@@ -384,10 +487,12 @@ void seq_latent_kv_store(torch::Tensor dkv, int64_t rank, torch::Tensor norm_w,
 // ------------------------------------------------------- gated activations
 // mode 0: silu(a) * b   mode 1: sigmoid(a) * b   mode 2: tanh(a)
 // mode 3: gelu(a), the exact (erf) form
+// mode 4: g * sigmoid(p1 * g) * (u + p2), g = min(a, p0), u = clamp(b, +-p0)
 template <typename T>
 __global__ void act_mul_kernel(T* __restrict__ out, const T* __restrict__ a,
                                long lda, const T* __restrict__ b, long ldb,
-                               long rows, int cols, int mode) {
+                               long rows, int cols, int mode, float p0,
+                               float p1, float p2) {
   long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
   const long stride = (long)gridDim.x * blockDim.x;
   const long n = rows * cols;
@@ -400,6 +505,10 @@ __global__ void act_mul_kernel(T* __restrict__ out, const T* __restrict__ a,
       v = tanhf(av);
     } else if (mode == 3) {
       v = gelu_erff_acc(av);
+    } else if (mode == 4) {
+      const float g = fminf(av, p0);
+      const float u = fminf(fmaxf(ldf(b + r * ldb + c), -p0), p0);
+      v = g * sigmoidf_acc(p1 * g) * (u + p2);
     } else {
       const float bv = ldf(b + r * ldb + c);
       v = (mode == 0 ? siluf_acc(av) : sigmoidf_acc(av)) * bv;
@@ -409,7 +518,7 @@ __global__ void act_mul_kernel(T* __restrict__ out, const T* __restrict__ a,
 }
 
 void seq_act_mul(torch::Tensor out, torch::Tensor a, torch::Tensor b,
-                 int64_t mode) {
+                 int64_t mode, double p0, double p1, double p2) {
   CHECK_ROWS(a);
   CHECK_ROWS(b);
   TORCH_CHECK(a.sizes() == b.sizes() && out.is_contiguous() &&
@@ -423,7 +532,8 @@ void seq_act_mul(torch::Tensor out, torch::Tensor a, torch::Tensor b,
   auto stream = at::hip::getCurrentHIPStream();
   SEQ_DISPATCH_T(a.scalar_type(), { hipLaunchKernelGGL((act_mul_kernel<T>), dim3(nblk), dim3(256), 0, stream, 
       (T*)out.data_ptr(), (const T*)a.data_ptr(), a.stride(0),
-      (const T*)b.data_ptr(), b.stride(0), rows, cols, (int)mode); });
+      (const T*)b.data_ptr(), b.stride(0), rows, cols, (int)mode, (float)p0,
+      (float)p1, (float)p2); });
   HIP_CHECK_KERNEL();
 }
 

@@ -2,6 +2,7 @@
 // and decode tokens alike (a decode token is a portion of length 1):
 //
 //   delta rule : S <- diag(w) S - (a*u)(u^T S) + k v^T ,  o = S^T r
+//   gated linear attention: S <- diag(w) S + k v^T     ,  o = S^T q
 //   state space: S <- exp(-exp(A) dt) S + dt B x^T     ,  y = S^T C + D x
 //
 // State columns are independent in both recurrences, so the state matrix
@@ -16,7 +17,8 @@
 // Per-token inputs of a lane's rows are contiguous and come in with 16-byte
 // loads when the layout allows (scalar loads otherwise); the inputs of token
 // t+1 are requested before the arithmetic of token t.  The delta rule's
-// decay and removal rate cost three exponentials per row: the 16 column
+// decay and removal rate cost three exponentials per row (gated linear
+// attention's decay an exponential and a logarithm): the 16 column
 // lanes of a row group would all compute the same ones, so each computes
 // one sixteenth and the group exchanges them by lane shuffles.
 // All state math is fp32 for bf16 or fp32 inputs.
@@ -230,6 +232,152 @@ void seq_delta_rule(torch::Tensor out, torch::Tensor r, torch::Tensor k,
     else if (rpl <= 16) DELTA_LAUNCH(16);
     else if (rpl <= 32) DELTA_LAUNCH(32);
     else DELTA_LAUNCH(64);
+  });
+  HIP_CHECK_KERNEL();
+}
+
+// ------------------------------------------------- gated linear attention
+// decay of key channel i: sigmoid(z_i + zb_i)^(1/tau)
+//   = exp(inv_tau * log_sigmoid(z_i + zb_i)), fp32
+template <int RPL>
+struct GlaIn {
+  static constexpr int NC = (RPL + 15) / 16;   // rows whose decay I compute
+  float q[RPL], k[RPL];
+  float zl[NC];
+  float v;
+};
+
+template <typename T, int RPL>
+DEV_INLINE void gla_load(GlaIn<RPL>& in, const T* q, const T* k, const T* v,
+                         const T* zl, long ldq, long ldk, long ldv, long ldz,
+                         long n, int hoff_k, int row0, int Dk, int vcol,
+                         bool colok, int ci, bool vec) {
+  load_rows<T, RPL>(in.q, q + n * ldq + hoff_k + row0, row0, Dk, vec);
+  load_rows<T, RPL>(in.k, k + n * ldk + hoff_k + row0, row0, Dk, vec);
+#pragma unroll
+  for (int c = 0; c < GlaIn<RPL>::NC; ++c) {
+    const int i = ci + 16 * c;
+    const bool ok = i < RPL && row0 + i < Dk;
+    in.zl[c] = ok ? ldf(zl + n * ldz + hoff_k + row0 + i) : 0.f;
+  }
+  in.v = colok ? ldf(v + n * ldv + vcol) : 0.f;
+}
+
+template <typename T, int RPL>
+__global__ __launch_bounds__(256) void gla_scan_kernel(
+    float* __restrict__ out,            // (N, H*Dv) fp32, un-normalised o
+    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
+    const T* __restrict__ zl, long ldq, long ldk, long ldv, long ldz,
+    const float* __restrict__ z_bias, float* __restrict__ state,
+    const int* __restrict__ cu_q, const int* __restrict__ state_slot, int H,
+    int Dk, int Dv, float q_scale, float inv_tau, bool vec) {
+  constexpr int NC = GlaIn<RPL>::NC;
+  const int cblocks = (Dv + 63) / 64;
+  const int b = blockIdx.x / (H * cblocks);
+  const int h = (blockIdx.x / cblocks) % H;
+  const int cb = blockIdx.x % cblocks;
+  const int lane = threadIdx.x & 63;
+  const int wid = threadIdx.x >> 6;
+  const int ci = lane / RG;                       // column index in the wave
+  const int col = cb * 64 + wid * COLS_PER_WAVE + ci;
+  const int rg = lane % RG;
+  const int row0 = rg * RPL;
+  const bool colok = col < Dv;
+  const int q0 = cu_q[b], q1 = cu_q[b + 1];
+  if (q1 <= q0) return;
+  // a whole wave past the last column has nothing to do (wave-uniform)
+  if (cb * 64 + wid * COLS_PER_WAVE >= Dv) return;
+
+  float* S = state + (((long)state_slot[b] * H + h) * Dk) * Dv;
+  float s[RPL], zbc[NC];
+#pragma unroll
+  for (int i = 0; i < RPL; ++i) {
+    const int row = row0 + i;
+    s[i] = (colok && row < Dk) ? S[(long)row * Dv + col] : 0.f;
+  }
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const int i = ci + 16 * c;
+    const bool ok = i < RPL && row0 + i < Dk;
+    zbc[c] = ok ? z_bias[h * Dk + row0 + i] : 0.f;
+  }
+  const int hoff_k = h * Dk;
+  const int vcol = h * Dv + col;
+
+  GlaIn<RPL> cur, nxt;
+  gla_load<T, RPL>(cur, q, k, v, zl, ldq, ldk, ldv, ldz, q0, hoff_k, row0, Dk,
+                   vcol, colok, ci, vec);
+  for (int n = q0; n < q1; ++n) {
+    if (n + 1 < q1)
+      gla_load<T, RPL>(nxt, q, k, v, zl, ldq, ldk, ldv, ldz, n + 1, hoff_k,
+                       row0, Dk, vcol, colok, ci, vec);
+    // my share of the decays: rows ci, ci+16, .. of this row group
+    float decm[NC];
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
+      decm[c] = expf(-inv_tau * softplusf_acc(-(cur.zl[c] + zbc[c])));
+    float o = 0.f;
+#pragma unroll
+    for (int i = 0; i < RPL; ++i) {
+      const int src = (i % 16) * RG + rg;          // lane that owns row i
+      const float dec = __shfl(decm[i / 16], src, WAVE_SIZE);
+      s[i] = dec * s[i] + cur.k[i] * cur.v;
+      o += s[i] * (cur.q[i] * q_scale);
+    }
+    o = lanegroup_sum<RG>(o);
+    if (colok && rg == 0) out[(long)n * H * Dv + vcol] = o;
+    cur = nxt;
+  }
+#pragma unroll
+  for (int i = 0; i < RPL; ++i) {
+    const int row = row0 + i;
+    if (colok && row < Dk) S[(long)row * Dv + col] = s[i];
+  }
+}
+
+#define GLA_LAUNCH(RPLV)                                                     \
+  hipLaunchKernelGGL((gla_scan_kernel<T, RPLV>), dim3(grid), dim3(256), 0,   \
+      stream, out.data_ptr<float>(), (const T*)q.data_ptr(),                 \
+      (const T*)k.data_ptr(), (const T*)v.data_ptr(),                        \
+      (const T*)z_lin.data_ptr(), q.stride(0), k.stride(0), v.stride(0),     \
+      z_lin.stride(0), z_bias.data_ptr<float>(), state.data_ptr<float>(),    \
+      cu_q.data_ptr<int>(), state_slot.data_ptr<int>(), H, Dk, Dv,           \
+      (float)q_scale, (float)inv_tau,                                        \
+      rows_vectorizable<T>(q, 0, Dk, RPLV) &&                                \
+          rows_vectorizable<T>(k, 0, Dk, RPLV))
+
+void seq_gla_scan(torch::Tensor out, torch::Tensor q, torch::Tensor k,
+                  torch::Tensor v, torch::Tensor z_lin, torch::Tensor z_bias,
+                  torch::Tensor state, torch::Tensor cu_q,
+                  torch::Tensor state_slot, double q_scale, double inv_tau) {
+  CHECK_ROWS(q); CHECK_ROWS(k); CHECK_ROWS(v); CHECK_ROWS(z_lin);
+  CHECK_F32(z_bias); CHECK_F32(state); CHECK_F32(out);
+  CHECK_I32(cu_q); CHECK_I32(state_slot);
+  TORCH_CHECK(state.dim() == 4);
+  const int H = state.size(1), Dk = state.size(2), Dv = state.size(3);
+  const long N = q.size(0);
+  TORCH_CHECK(q.size(1) == H * Dk && k.size(1) == H * Dk &&
+              z_lin.size(1) == H * Dk && v.size(1) == H * Dv,
+              "gated linear attention operand widths");
+  TORCH_CHECK(k.size(0) == N && v.size(0) == N && z_lin.size(0) == N &&
+              out.size(0) == N && out.size(1) == H * Dv);
+  TORCH_CHECK(z_bias.numel() == H * Dk);
+  auto dt = q.scalar_type();
+  TORCH_CHECK(k.scalar_type() == dt && v.scalar_type() == dt &&
+              z_lin.scalar_type() == dt);
+  TORCH_CHECK(Dk <= 256, "gated linear attention: key dim above 256 not supported");
+  const int B = state_slot.numel();
+  TORCH_CHECK(cu_q.numel() == B + 1);
+  if (N == 0 || B == 0) return;
+  const int grid = B * H * ((Dv + 63) / 64);
+  const int rpl = (Dk + RG - 1) / RG;
+  auto stream = at::hip::getCurrentHIPStream();
+  SEQ_DISPATCH_T(dt, {
+    if (rpl <= 4) GLA_LAUNCH(4);
+    else if (rpl <= 8) GLA_LAUNCH(8);
+    else if (rpl <= 16) GLA_LAUNCH(16);
+    else if (rpl <= 32) GLA_LAUNCH(32);
+    else GLA_LAUNCH(64);
   });
   HIP_CHECK_KERNEL();
 }

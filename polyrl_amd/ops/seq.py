@@ -1,8 +1,10 @@
 """Sequence-mixer ops for hybrid decoders: fp32-residual norms (plain and
-offset weights, fused joints), stateful causal convolutions, the generalised
-delta rule, the selective state-space scan, windowed latent attention with a
-softmax sink, grouped-query window attention over paged K/V rows, and
-table-routed or router-chosen expert feed-forwards.
+offset weights, fused joints, scaled branches), the composed embedding
+(scaled row + hashed pair row + sinusoid), stateful causal convolutions, the
+generalised delta rule, gated linear attention, the selective state-space
+scan, windowed latent attention with a softmax sink, grouped-query (window or
+causal) attention over paged K/V rows, and table-routed or router-chosen
+expert feed-forwards.
 
 Same policy as the rest of ``polyrl_amd.ops``: on a HIP device the in-tree
 extension is REQUIRED (csrc/seq_*.hip, templated on the activation type:
@@ -44,40 +46,84 @@ def _ext():
 def add_rmsnorm_f32res(res: torch.Tensor, y: Optional[torch.Tensor],
                        weight: torch.Tensor, eps: float,
                        out_dtype: torch.dtype,
-                       offset: float = 0.0) -> torch.Tensor:
-    """res (N, D) fp32 += y in place, then RMS-norm(res) * (offset + weight)
-    -> out_dtype.  ``weight`` holds one number (for all coordinates) or D."""
+                       offset: float = 0.0, scale: float = 1.0,
+                       extra: Optional[torch.Tensor] = None,
+                       extra_vec: Optional[torch.Tensor] = None
+                       ) -> torch.Tensor:
+    """res (N, D) fp32 += scale * y [+ extra (N, D) fp32] [+ extra_vec (D,)
+    fp32] in place, then RMS-norm(res) * (offset + weight) -> out_dtype.
+    ``weight`` holds one number (for all coordinates) or D."""
     if res.is_cuda:
         out = torch.empty(res.shape, dtype=out_dtype, device=res.device)
-        _ext().seq_add_rmsnorm(out, res, y if y is not None else torch.Tensor(),
-                               weight, eps, 0, offset, torch.Tensor())
+        e = torch.Tensor()
+        _ext().seq_add_rmsnorm(out, res, y if y is not None else e,
+                               weight, eps, 0, offset, e, scale,
+                               extra if extra is not None else e,
+                               extra_vec if extra_vec is not None else e)
         return out
-    return R.add_rmsnorm_f32res(res, y, weight, eps, out_dtype, offset)
+    return R.add_rmsnorm_f32res(res, y, weight, eps, out_dtype, offset, scale,
+                                extra, extra_vec)
 
 
 def residual_add_cast(res: torch.Tensor, y: Optional[torch.Tensor],
-                      out_dtype: torch.dtype) -> torch.Tensor:
-    """res += y in place; returns res in out_dtype (res itself for fp32)."""
+                      out_dtype: torch.dtype,
+                      scale: float = 1.0) -> torch.Tensor:
+    """res += scale * y in place; returns res in out_dtype (res itself for
+    fp32)."""
     if res.is_cuda:
         if y is None and out_dtype == torch.float32:
             return res
         out = res if out_dtype == torch.float32 else \
             torch.empty(res.shape, dtype=out_dtype, device=res.device)
-        _ext().seq_add_rmsnorm(out, res, y if y is not None else torch.Tensor(),
-                               torch.Tensor(), 0.0, 1, 0.0, torch.Tensor())
+        e = torch.Tensor()
+        _ext().seq_add_rmsnorm(out, res, y if y is not None else e,
+                               e, 0.0, 1, 0.0, e, scale, e, e)
         return out
-    return R.residual_add_cast(res, y, out_dtype)
+    return R.residual_add_cast(res, y, out_dtype, scale)
 
 
 def add_scaled_unit_rms(res: torch.Tensor, y: torch.Tensor,
                         weight: torch.Tensor, eps: float,
-                        offset: float = 0.0) -> None:
-    """res += y / rms(y) * (offset + weight), in place (weight (D,) fp32)."""
+                        offset: float = 0.0, scale: float = 1.0) -> None:
+    """res += scale * y / rms(y) * (offset + weight), in place (weight (D,)
+    fp32)."""
     if res.is_cuda:
-        _ext().seq_add_rmsnorm(res, res, y, weight, eps, 2, offset,
-                               torch.Tensor())
+        e = torch.Tensor()
+        _ext().seq_add_rmsnorm(res, res, y, weight, eps, 2, offset, e, scale,
+                               e, e)
         return
-    R.add_scaled_unit_rms(res, y, weight, eps, offset)
+    R.add_scaled_unit_rms(res, y, weight, eps, offset, scale)
+
+
+def sinusoid_inv_freq(width: int, base: float, device) -> torch.Tensor:
+    """f_i = base^(-2i/width) for the ceil(width/2) sin/cos pairs of a
+    position vector, rounded once to fp32."""
+    i = torch.arange((width + 1) // 2, dtype=torch.float64)
+    return (base ** (-2.0 * i / width)).float().to(device)
+
+
+def embed_compose(table, tokens, scale: float, pair_table, prev_tokens,
+                  mul_prev: int, mul_cur: int, buckets: int, positions,
+                  inv_freq) -> torch.Tensor:
+    """The fp32 embedding output (N, D): table[token] * scale
+    [+ pair_table[(prev * mul_prev + token * mul_cur) mod buckets], row
+    ``buckets`` where prev < 0 (a sequence's first token)]
+    [+ the sinusoid of the position: entry 2i = sin(fp32(p) * inv_freq[i]),
+    entry 2i+1 = cos of the same angle]."""
+    if table.is_cuda:
+        out = torch.empty(tokens.shape[0], table.shape[1],
+                          dtype=torch.float32, device=table.device)
+        if tokens.shape[0]:
+            e = torch.Tensor()
+            _ext().seq_embed_compose(
+                out, table, tokens, scale,
+                pair_table if pair_table is not None else e,
+                prev_tokens if pair_table is not None else e,
+                mul_prev, mul_cur, buckets, positions,
+                inv_freq if inv_freq is not None else e)
+        return out
+    return R.embed_compose(table, tokens, scale, pair_table, prev_tokens,
+                           mul_prev, mul_cur, buckets, positions, inv_freq)
 
 
 def add_unit_rms_then_norm(res: torch.Tensor, y: torch.Tensor,
@@ -89,7 +135,9 @@ def add_unit_rms_then_norm(res: torch.Tensor, y: torch.Tensor,
     res / rms(res) * (offset + w_next) as out_dtype."""
     if res.is_cuda:
         out = torch.empty(res.shape, dtype=out_dtype, device=res.device)
-        _ext().seq_add_rmsnorm(out, res, y, w_post, eps, 3, offset, w_next)
+        e = torch.Tensor()
+        _ext().seq_add_rmsnorm(out, res, y, w_post, eps, 3, offset, w_next,
+                               1.0, e, e)
         return out
     return R.add_unit_rms_then_norm(res, y, w_post, w_next, eps, out_dtype,
                                     offset)
@@ -132,7 +180,7 @@ def delta_rule(r, k, v, w_lin, a_lin, g, w0, a_bias, norm_w, state, cu_q,
             _ext().seq_delta_rule(o, r, k, v, w_lin, a_lin, w0, a_bias, state,
                                   cu_q, state_slot, decay_scale, key_eps)
             # per-head unit RMS, plain weight, sigmoid output gate
-            _ext().seq_group_rmsnorm(out, o, norm_w, H, eps, g)
+            _ext().seq_group_rmsnorm(out, o, norm_w, H, eps, g, 1)
         return out
     return R.delta_rule(r, k, v, w_lin, a_lin, g, w0, a_bias, norm_w, state,
                         cu_q, state_slot, decay_scale, key_eps, eps, out_dtype)
@@ -155,16 +203,39 @@ def ssm_scan(xbc, dt, z, dt_bias, a_log, d_skip, state, cu_q, state_slot,
                       state_slot, groups)
 
 
-def group_rmsnorm(y, weight, groups: int, eps: float, out_dtype):
+def group_rmsnorm(y, weight, groups: int, eps: float, out_dtype,
+                  gate=None, gate_act: str = "sigmoid"):
     """RMS-norm each of ``groups`` equal parts of a row by its own root mean
-    square, times weight (D,)."""
+    square, times weight ((D,), or (D/groups,) shared by the groups), times
+    sigmoid(gate) or silu(gate) when a gate (N, D) is given."""
     if y.is_cuda:
         out = torch.empty(y.shape, dtype=out_dtype, device=y.device)
         if y.shape[0]:
-            _ext().seq_group_rmsnorm(out, y, weight, groups, eps,
-                                     torch.Tensor())
+            _ext().seq_group_rmsnorm(
+                out, y, weight, groups, eps,
+                gate if gate is not None else torch.Tensor(),
+                {"sigmoid": 1, "silu": 2}[gate_act])
         return out
-    return R.group_rmsnorm(y, weight, groups, eps, out_dtype)
+    return R.group_rmsnorm(y, weight, groups, eps, out_dtype, gate, gate_act)
+
+
+def gla_scan(q, k, v, z_lin, z_bias, state, cu_q, state_slot,
+             q_scale: float, inv_tau: float) -> torch.Tensor:
+    """Gated linear attention over packed rows; ``state`` (slots, H, Dk, Dv)
+    fp32 in place.  Per head: decay = exp(log_sigmoid(z_lin + z_bias) *
+    inv_tau) per key channel, S <- diag(decay) S + k v^T,
+    o = S^T (q * q_scale).  Returns o as fp32 (N, H*Dv), not normed.
+    Inputs may be column slices."""
+    if q.is_cuda:
+        slots, H, Dk, Dv = state.shape
+        out = torch.empty(q.shape[0], H * Dv, dtype=torch.float32,
+                          device=q.device)
+        if q.shape[0]:
+            _ext().seq_gla_scan(out, q, k, v, z_lin, z_bias, state, cu_q,
+                                state_slot, q_scale, inv_tau)
+        return out
+    return R.gla_scan(q, k, v, z_lin, z_bias, state, cu_q, state_slot,
+                      q_scale, inv_tau)
 
 
 def rope_inv_freq(dims: int, base: float, device) -> torch.Tensor:
@@ -270,13 +341,17 @@ def gqa_prepare_store(q, k, v, q_norm, k_norm, eps: float, inv_freq,
 def gqa_window_attention(q, cache, page_table, seq_of_tok, positions, H: int,
                          G: int, D: int, Dv: int, window: int,
                          keep_first: int, rel, dist_bucket, gate,
-                         scale: float, out_dtype, tiles=None) -> torch.Tensor:
+                         scale: float, out_dtype, tiles=None, sink=None,
+                         q_temp_coef: float = 0.0,
+                         q_temp_every: int = 1) -> torch.Tensor:
     """Softmax attention of every row against its sequence's paged K/V rows
     (layout of :func:`gqa_prepare_store`).  Row at position p sees key j if
     j <= p and (p - j < window or j < keep_first).  score = q.k * scale
-    [+ rel[dist_bucket[p - j], head]]; ``gate`` (N, H) multiplies head h's
-    output by sigmoid(gate[n, h]).  Query head h reads key/value head
-    h // (H // G).  Returns (N, H*Dv)."""
+    * (1 + q_temp_coef * ln(floor((p + 1) / q_temp_every) + 1))
+    [+ rel[dist_bucket[p - j], head]]; with ``sink`` (H,) fp32 the
+    denominator also holds exp(sink[h]) once; ``gate`` (N, H) multiplies
+    head h's output by sigmoid(gate[n, h]).  Query head h reads key/value
+    head h // (H // G).  Returns (N, H*Dv)."""
     if q.is_cuda:
         out = torch.empty(q.shape[0], H * Dv, dtype=out_dtype,
                           device=q.device)
@@ -285,7 +360,9 @@ def gqa_window_attention(q, cache, page_table, seq_of_tok, positions, H: int,
             args = (cache, page_table, seq_of_tok, positions, H, G, D, Dv,
                     window, keep_first, rel if rel is not None else e,
                     dist_bucket if dist_bucket is not None else e,
-                    gate if gate is not None else e, scale)
+                    gate if gate is not None else e, scale,
+                    sink if sink is not None else e, q_temp_coef,
+                    q_temp_every)
             if tiles is not None and tiles[2] == 0 and \
                     gqa_mfma_supported(q, D, Dv):
                 _ext().seq_gqa_window_attention_mfma(out, q, tiles[0],
@@ -295,7 +372,8 @@ def gqa_window_attention(q, cache, page_table, seq_of_tok, positions, H: int,
         return out
     return R.gqa_window_attention(q, cache, page_table, seq_of_tok, positions,
                                   H, G, D, Dv, window, keep_first, rel,
-                                  dist_bucket, gate, scale, out_dtype)
+                                  dist_bucket, gate, scale, out_dtype, sink,
+                                  q_temp_coef, q_temp_every)
 
 
 def gqa_mfma_supported(q, D: int, Dv: int) -> bool:
@@ -327,7 +405,7 @@ def gelu_erf(x):
     if x.is_cuda:
         out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
         if x.shape[0]:
-            _ext().seq_act_mul(out, x, x, 3)
+            _ext().seq_act_mul(out, x, x, 3, 0.0, 0.0, 0.0)
         return out
     return R.gelu_erf(x)
 
@@ -373,9 +451,20 @@ def silu_mul_any(gate, up):
     if gate.is_cuda:
         out = torch.empty(gate.shape, dtype=gate.dtype, device=gate.device)
         if gate.shape[0]:
-            _ext().seq_act_mul(out, gate, up, 0)
+            _ext().seq_act_mul(out, gate, up, 0, 0.0, 0.0, 0.0)
         return out
     return R.silu_mul_any(gate, up)
+
+
+def clamped_glu(gate, up, limit: float, slope: float, shift: float):
+    """g * sigmoid(slope * g) * (u + shift) with g = min(gate, limit) and
+    u = clamp(up, -limit, limit) (row-strided views allowed)."""
+    if gate.is_cuda:
+        out = torch.empty(gate.shape, dtype=gate.dtype, device=gate.device)
+        if gate.shape[0]:
+            _ext().seq_act_mul(out, gate, up, 4, limit, slope, shift)
+        return out
+    return R.clamped_glu(gate, up, limit, slope, shift)
 
 
 def sigmoid_mul(x, gate):
@@ -383,7 +472,7 @@ def sigmoid_mul(x, gate):
     if x.is_cuda:
         out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
         if x.shape[0]:
-            _ext().seq_act_mul(out, gate, x, 1)
+            _ext().seq_act_mul(out, gate, x, 1, 0.0, 0.0, 0.0)
         return out
     return R.sigmoid_mul(x, gate)
 
@@ -393,7 +482,7 @@ def tanh_act(x):
     if x.is_cuda:
         out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
         if x.shape[0]:
-            _ext().seq_act_mul(out, x, x, 2)
+            _ext().seq_act_mul(out, x, x, 2, 0.0, 0.0, 0.0)
         return out
     return R.tanh_act(x)
 

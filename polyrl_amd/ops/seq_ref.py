@@ -16,23 +16,29 @@ def _w(weight: torch.Tensor) -> torch.Tensor:
     return weight.float().reshape(-1)
 
 
-def add_rmsnorm_f32res(res, y, weight, eps, out_dtype, offset=0.0):
+def add_rmsnorm_f32res(res, y, weight, eps, out_dtype, offset=0.0,
+                       scale=1.0, extra=None, extra_vec=None):
     if y is not None:
-        res.add_(y.float())
+        res.add_(y.float() * scale if scale != 1.0 else y.float())
+    if extra is not None:
+        res.add_(extra)
+    if extra_vec is not None:
+        res.add_(extra_vec.float())
     inv = torch.rsqrt(res.pow(2).mean(-1, keepdim=True) + eps)
     return (res * inv * (_w(weight) + offset)).to(out_dtype)
 
 
-def residual_add_cast(res, y, out_dtype):
+def residual_add_cast(res, y, out_dtype, scale=1.0):
     if y is not None:
-        res.add_(y.float())
+        res.add_(y.float() * scale if scale != 1.0 else y.float())
     return res if out_dtype == torch.float32 else res.to(out_dtype)
 
 
-def add_scaled_unit_rms(res, y, weight, eps, offset=0.0):
+def add_scaled_unit_rms(res, y, weight, eps, offset=0.0, scale=1.0):
     yf = y.float()
     inv = torch.rsqrt(yf.pow(2).mean(-1, keepdim=True) + eps)
-    res.add_(yf * inv * (_w(weight) + offset))
+    add = yf * inv * (_w(weight) + offset)
+    res.add_(add * scale if scale != 1.0 else add)
 
 
 def add_unit_rms_then_norm(res, y, w_post, w_next, eps, out_dtype, offset):
@@ -124,11 +130,64 @@ def ssm_scan(xbc, dt, z, dt_bias, a_log, d_skip, state, cu_q, state_slot,
     return y.view(N, inner) * (zf * torch.sigmoid(zf))
 
 
-def group_rmsnorm(y, weight, groups, eps, out_dtype):
+def group_rmsnorm(y, weight, groups, eps, out_dtype, gate=None,
+                  gate_act="sigmoid"):
     N, D = y.shape
     yf = y.float().view(N, groups, D // groups)
     yf = yf * torch.rsqrt(yf.pow(2).mean(-1, keepdim=True) + eps)
-    return (yf.view(N, D) * weight.float()).to(out_dtype)
+    wf = weight.float()
+    if wf.numel() != D:                      # one weight row for all groups
+        wf = wf.repeat(groups)
+    out = yf.view(N, D) * wf
+    if gate is not None:
+        gf = gate.float()
+        out = out * (torch.sigmoid(gf) if gate_act == "sigmoid"
+                     else gf * torch.sigmoid(gf))
+    return out.to(out_dtype)
+
+
+def embed_compose(table, tokens, scale, pair_table, prev_tokens, mul_prev,
+                  mul_cur, buckets, positions, inv_freq):
+    x = table[tokens.long()].float() * scale
+    if pair_table is not None:
+        prev, cur = prev_tokens.long(), tokens.long()
+        row = torch.where(prev < 0, torch.full_like(cur, buckets),
+                          (prev.clamp(min=0) * mul_prev + cur * mul_cur)
+                          % buckets)
+        x = x + pair_table[row].float()
+    if inv_freq is not None:
+        D = table.shape[1]
+        ang = positions.float().unsqueeze(-1) * inv_freq.float()
+        pe = torch.stack([torch.sin(ang), torch.cos(ang)], -1)
+        x = x + pe.reshape(x.shape[0], -1)[:, :D]
+    return x
+
+
+def gla_scan(q, k, v, z_lin, z_bias, state, cu_q, state_slot, q_scale,
+             inv_tau):
+    slots, H, Dk, Dv = state.shape
+    N = q.shape[0]
+    qf = q.float().view(N, H, Dk) * q_scale
+    kf = k.float().view(N, H, Dk)
+    vf = v.float().view(N, H, Dv)
+    dec = torch.exp(torch.nn.functional.logsigmoid(
+        z_lin.float() + z_bias.float()) * inv_tau).view(N, H, Dk)
+    out = torch.empty(N, H * Dv, dtype=torch.float32, device=q.device)
+    cu = cu_q.tolist()
+    for b, slot in enumerate(state_slot.tolist()):
+        S = state[slot]                                  # (H, Dk, Dv)
+        for n in range(cu[b], cu[b + 1]):
+            S = dec[n].unsqueeze(-1) * S \
+                + kf[n].unsqueeze(-1) * vf[n].unsqueeze(1)
+            out[n] = torch.einsum("hk,hkv->hv", qf[n], S).reshape(-1)
+        state[slot] = S
+    return out
+
+
+def clamped_glu(gate, up, limit, slope, shift):
+    g = gate.float().clamp(max=limit)
+    u = up.float().clamp(-limit, limit)
+    return (g * torch.sigmoid(slope * g) * (u + shift)).to(gate.dtype)
 
 
 def _rotate(x, positions, inv_freq):
@@ -254,7 +313,8 @@ def gqa_prepare_store(q, k, v, q_norm, k_norm, eps, inv_freq, amp, positions,
 
 def gqa_window_attention(q, cache, page_table, seq_of_tok, positions, H, G,
                          D, Dv, window, keep_first, rel, dist_bucket, gate,
-                         scale, out_dtype):
+                         scale, out_dtype, sink=None, q_temp_coef=0.0,
+                         q_temp_every=1):
     N = q.shape[0]
     ps = cache.shape[1]
     flat = cache.view(-1, cache.shape[-1]).float()
@@ -270,11 +330,20 @@ def gqa_window_attention(q, cache, page_table, seq_of_tok, positions, H, G,
         kv = flat[rows]
         kk = kv[:, :G * D].view(-1, G, D).repeat_interleave(per, 1)
         vv = kv[:, G * D:].view(-1, G, Dv).repeat_interleave(per, 1)
-        s = torch.einsum("hd,jhd->hj", qf[n], kk) * scale
+        sc = scale
+        if q_temp_coef != 0.0:
+            sc = scale * (1.0 + q_temp_coef
+                          * math.log((p + 1) // q_temp_every + 1))
+        s = torch.einsum("hd,jhd->hj", qf[n], kk) * sc
         if rel is not None:
             dist = torch.tensor([p - j for j in js], dtype=torch.long)
             s = s + rel.float()[dist_bucket.long()[dist]].t()
-        o = torch.einsum("hj,jhv->hv", torch.softmax(s, -1), vv)
+        if sink is not None:
+            pr = torch.softmax(
+                torch.cat([s, sink.float().view(H, 1)], 1), -1)[:, :-1]
+        else:
+            pr = torch.softmax(s, -1)
+        o = torch.einsum("hj,jhv->hv", pr, vv)
         if gate is not None:
             o = o * torch.sigmoid(gate[n].float()).unsqueeze(-1)
         out[n] = o

@@ -794,9 +794,19 @@ class Engine:
         from .hybrid_model import HybridBatch
         dev = self.device
         tok, pos, sot, cu, slots, sids, maps = [], [], [], [0], [], [], []
+        prev = []
         for b, (r, start, toks) in enumerate(items):
             sid = self._seq_ids[r.rid]
             n = len(toks)
+            # the token before each row: the request's own history for the
+            # portion's first row (-1 at the start of the sequence)
+            if start == 0:
+                prev.append(-1)
+            elif start - 1 < len(r.input_ids):
+                prev.append(r.input_ids[start - 1])
+            else:
+                prev.append(r.output_ids[start - 1 - len(r.input_ids)])
+            prev.extend(toks[:-1])
             tok.extend(toks)
             pos.extend(range(start, start + n))
             sot.extend([b] * n)
@@ -808,6 +818,7 @@ class Engine:
         th = np.asarray(tok, dtype=np.int64)
         return HybridBatch(
             tokens=torch.from_numpy(th).to(dev), tokens_host=th,
+            prev_tokens=torch.tensor(prev, dtype=torch.int64, device=dev),
             positions=i32(pos), seq_of_tok=i32(sot), cu_q=i32(cu),
             state_slot=i32(slots),
             slot_mapping=torch.cat(maps).to(dev),

@@ -32,6 +32,7 @@ class HybridBatch:
     tokens at positions start[b]...; device tensors are int32 unless said."""
     tokens: torch.Tensor          # (N,) int64
     tokens_host: np.ndarray       # (N,) int64
+    prev_tokens: torch.Tensor     # (N,) int64, -1 at a sequence's first token
     positions: torch.Tensor       # (N,)
     seq_of_tok: torch.Tensor      # (N,)
     cu_q: torch.Tensor            # (B+1,)
@@ -52,8 +53,12 @@ def set_tuned_products(on: bool) -> None:
     _TUNED = bool(on)
 
 
-def _mm(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
-    """y = x @ w.T (vendor matrix product, fp32 accumulation)."""
+def _mm(x: torch.Tensor, w: torch.Tensor,
+        b: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """y = x @ w.T [+ b] (vendor matrix product, fp32 accumulation; the
+    bias joins the accumulator before the result is rounded)."""
+    if b is not None:
+        return torch.addmm(b, x, w.t())
     if _TUNED and x.is_cuda and x.dtype == torch.bfloat16 \
             and x.shape[0] <= 512 and x.is_contiguous() \
             and w.shape[0] >= 64 and w.shape[1] >= 64:
@@ -106,6 +111,52 @@ class DeltaRuleMixer(_Part):
                            states.tensors[(li, "S")], bt.cu_q, bt.state_slot,
                            s.decay_scale, s.key_eps, model.cfg.norm_eps,
                            h.dtype)
+        return _mm(y, self.wo)
+
+
+class GLAMixer(_Part):
+    """Gated linear attention (models.hybrid.GLASpec): one fused projection
+    for queries, keys, values, the output gate and the low-rank decay input;
+    the scan keeps one fp32 (dim, vdim) state per head and sequence; the
+    per-head RMS norm (one weight row shared by the heads) and the SiLU
+    output gate are one kernel."""
+
+    def __init__(self, spec, width, device, dtype):
+        self.spec = s = spec
+        self.nk, self.nv = s.heads * s.dim, s.heads * s.vdim
+        self.rank = int(s.decay_rank)
+        z = lambda *a, dt=dtype: torch.empty(*a, device=device, dtype=dt)
+        f32 = torch.float32
+        self.w_in = z(2 * self.nk + 2 * self.nv + self.rank, width)
+        self.a2 = z(self.nk, self.rank)
+        self.a2_b = z(self.nk, dt=f32)
+        self.norm = z(s.vdim, dt=f32)
+        self.wo = z(width, self.nv)
+
+    def named(self, p):
+        nk, nv = self.nk, self.nv
+        return {p + "q": self.w_in[:nk], p + "k": self.w_in[nk:2 * nk],
+                p + "v": self.w_in[2 * nk:2 * nk + nv],
+                p + "g": self.w_in[2 * nk + nv:2 * nk + 2 * nv],
+                p + "a1": self.w_in[2 * nk + 2 * nv:],
+                p + "a2": self.a2, p + "a2.b": self.a2_b,
+                p + "norm": self.norm, p + "o": self.wo}
+
+    def state_shapes(self):
+        s = self.spec
+        return {"S": (s.heads, s.dim, s.vdim)}
+
+    def forward(self, h, bt, li, model, cache, states):
+        s, nk, nv = self.spec, self.nk, self.nv
+        proj = _mm(h, self.w_in)
+        z_lin = _mm(proj.narrow(1, 2 * nk + 2 * nv, self.rank), self.a2)
+        o = seq.gla_scan(proj.narrow(1, 0, nk), proj.narrow(1, nk, nk),
+                         proj.narrow(1, 2 * nk, nv), z_lin, self.a2_b,
+                         states.tensors[(li, "S")], bt.cu_q, bt.state_slot,
+                         s.dim ** -0.5, 1.0 / s.tau)
+        y = seq.group_rmsnorm(o, self.norm, s.heads, model.cfg.norm_eps,
+                              h.dtype, gate=proj.narrow(1, 2 * nk + nv, nv),
+                              gate_act="silu")
         return _mm(y, self.wo)
 
 
@@ -227,6 +278,11 @@ class WindowAttnMixer(_Part):
         self.ng = s.heads if s.head_gate else 0
         self.row = s.kv_heads * (s.dim + s.vdim)
         self.w_in = z(self.nq + self.nk + self.nv + self.ng, width)
+        self.b_in = z(self.nq + self.nk + self.nv + self.ng) \
+            if s.qkv_bias else None
+        if self.b_in is not None:
+            self.b_in.zero_()             # the head gate has no bias
+        self.sink = z(s.heads, dt=f32) if s.sink else None
         self.q_norm = z(self.nq, dt=f32) if s.qk_norm else None
         self.k_norm = z(self.nk, dt=f32) if s.qk_norm else None
         self.wo = z(width, s.heads * s.vdim)
@@ -254,12 +310,19 @@ class WindowAttnMixer(_Part):
             out[p + "k.norm"] = self.k_norm
         if self.rel is not None:
             out[p + "rel"] = self.rel
+        if self.b_in is not None:
+            out[p + "q.b"] = self.b_in[:a]
+            out[p + "k.b"] = self.b_in[a:b]
+            if self.nv:
+                out[p + "v.b"] = self.b_in[b:b + self.nv]
+        if self.sink is not None:
+            out[p + "sink"] = self.sink
         return out
 
     def forward(self, h, bt, li, model, cache, states):
         s = self.spec
         a, b = self.nq, self.nq + self.nk
-        proj = _mm(h, self.w_in)
+        proj = _mm(h, self.w_in, self.b_in)
         rows = cache.rows[li]
         q = seq.gqa_prepare_store(
             proj.narrow(1, 0, a), proj.narrow(1, a, self.nk),
@@ -272,25 +335,44 @@ class WindowAttnMixer(_Part):
             s.kv_heads, s.dim, s.vdim, s.window, s.keep_first, self.rel,
             self.dist_bucket,
             proj.narrow(1, b + self.nv, self.ng) if self.ng else None,
-            s.scale, h.dtype, tiles=bt.attn_tiles)
+            s.scale, h.dtype, tiles=bt.attn_tiles, sink=self.sink,
+            q_temp_coef=s.q_temp_coef, q_temp_every=s.q_temp_every)
         return _mm(o, self.wo)
 
 
 class DenseFF(_Part):
+    """Gated feed-forward, gate and up as one product: silu(gate) * up, or
+    the clamped form (models.hybrid.FFSpec.act); optional biases."""
+
     def __init__(self, spec, width, vocab, device, dtype):
+        self.spec = spec
         self.ff = spec.ff
         self.w_gu = torch.empty(2 * spec.ff, width, device=device, dtype=dtype)
         self.w_down = torch.empty(width, spec.ff, device=device, dtype=dtype)
+        self.b_gu = self.b_down = None
+        if spec.bias:
+            self.b_gu = torch.empty(2 * spec.ff, device=device, dtype=dtype)
+            self.b_down = torch.empty(width, device=device, dtype=dtype)
 
     def named(self, p):
-        return {p + "gate": self.w_gu[:self.ff], p + "up": self.w_gu[self.ff:],
-                p + "down": self.w_down}
+        out = {p + "gate": self.w_gu[:self.ff], p + "up": self.w_gu[self.ff:],
+               p + "down": self.w_down}
+        if self.b_gu is not None:
+            out.update({p + "gate.b": self.b_gu[:self.ff],
+                        p + "up.b": self.b_gu[self.ff:],
+                        p + "down.b": self.b_down})
+        return out
 
     def forward(self, h, res, bt):
-        gu = _mm(h, self.w_gu)
-        act = seq.silu_mul_any(gu.narrow(1, 0, self.ff),
-                               gu.narrow(1, self.ff, self.ff))
-        return _mm(act, self.w_down)      # added by the caller's next norm
+        f = self.spec
+        gu = _mm(h, self.w_gu, self.b_gu)
+        gate, up = gu.narrow(1, 0, self.ff), gu.narrow(1, self.ff, self.ff)
+        if f.act == "clamped":
+            act = seq.clamped_glu(gate, up, f.limit, f.gate_slope, f.up_shift)
+        else:
+            act = seq.silu_mul_any(gate, up)
+        # added by the caller's next norm
+        return _mm(act, self.w_down, self.b_down)
 
 
 class TableMoE(_Part):
@@ -441,6 +523,7 @@ class RoutedMoE(_Part):
 
 
 _MIXERS = {"general_delta": DeltaRuleMixer, "mamba2": SSMMixer,
+           "gla": GLAMixer,
            "latent_attention": LatentAttnMixer, "attention": WindowAttnMixer}
 _FFS = {"dense": DenseFF, "moe": TableMoE, "routed_moe": RoutedMoE}
 
@@ -499,6 +582,38 @@ class SandwichLayer:
         return out
 
 
+class PreNormLayer:
+    """x += m * mixer(norm1(x)), x += m * ff(norm2(x)), then the token-side
+    input (also times m); per-channel norm weights."""
+
+    def __init__(self, cfg: HybridConfig, li: int, device, dtype):
+        L = cfg.layers[li]
+        W = cfg.hidden_size
+        f32 = torch.float32
+        self.norm1 = torch.empty(W, device=device, dtype=f32)
+        self.mixer = _MIXERS[L.mixer.kind](L.mixer, W, device, dtype)
+        self.ff = None if L.ff is None else \
+            _FFS[L.ff.kind](L.ff, W, cfg.vocab_size, device, dtype)
+        self.norm2 = torch.empty(W, device=device, dtype=f32) \
+            if self.ff is not None else None
+        d = cfg.token_side_dim
+        self.side_gate = torch.empty(d, W, device=device, dtype=dtype)
+        self.side_proj = torch.empty(W, d, device=device, dtype=dtype)
+        self.side_norm = torch.empty(W, device=device, dtype=f32)
+
+    def named(self, p: str) -> Dict[str, torch.Tensor]:
+        out = {p + "norm1": self.norm1}
+        if self.side_gate.shape[0] > 0:
+            out.update({p + "side.gate": self.side_gate,
+                        p + "side.proj": self.side_proj,
+                        p + "side.norm": self.side_norm})
+        out.update(self.mixer.named(p + "mix."))
+        if self.ff is not None:
+            out[p + "norm2"] = self.norm2
+            out.update(self.ff.named(p + "mlp."))
+        return out
+
+
 class HybridInferenceModel:
     """Weights + packed forward of a hybrid decoder for the rollout engine
     (same weight-update surface as InferenceModel: ``_name_map``,
@@ -520,8 +635,13 @@ class HybridInferenceModel:
                     and L.mixer.bias_rows is None:
                 raise ValueError("the distance-bias table's rows come from "
                                  "the checkpoint: call resolve_shapes first")
+            if L.mixer.kind == "gla" and L.mixer.decay_rank is None:
+                raise ValueError("the decay projection's rank comes from "
+                                 "the checkpoint: call resolve_shapes first")
         self.sandwich = cfg.layer_style == "sandwich"
-        layer_cls = SandwichLayer if self.sandwich else HybridLayer
+        self.prenorm = cfg.layer_style == "prenorm"
+        layer_cls = SandwichLayer if self.sandwich else \
+            PreNormLayer if self.prenorm else HybridLayer
         self.layers = [layer_cls(cfg, li, device, dtype)
                        for li in range(cfg.num_hidden_layers)]
         self.runs = cfg.run_order()
@@ -530,8 +650,9 @@ class HybridInferenceModel:
         self.side_embed = torch.empty(
             cfg.vocab_size, cfg.num_hidden_layers * cfg.token_side_dim,
             device=device, dtype=dtype)
-        self.final_norm = torch.empty(W if self.sandwich else 1,
-                                      device=device, dtype=torch.float32)
+        self.final_norm = torch.empty(
+            W if self.sandwich or self.prenorm else 1,
+            device=device, dtype=torch.float32)
         self.lm_head = torch.empty(cfg.vocab_size, W, device=device,
                                    dtype=dtype)
         self._name_map: Dict[str, torch.Tensor] = {
@@ -539,6 +660,18 @@ class HybridInferenceModel:
             "head": self.lm_head}
         if cfg.token_side_dim > 0:
             self._name_map["side.embed"] = self.side_embed
+        self.pair_embed = self.loop_step = self.pos_inv_freq = None
+        if cfg.bigram is not None:
+            self.pair_embed = torch.empty(cfg.bigram.buckets + 1, W,
+                                          device=device, dtype=dtype)
+            self._name_map["bigram"] = self.pair_embed
+        if cfg.loop_step:
+            self.loop_step = torch.empty(cfg.loop[2], W, device=device,
+                                         dtype=torch.float32)
+            self._name_map["loop.step"] = self.loop_step
+        if cfg.sin_pos_base > 0:
+            self.pos_inv_freq = seq.sinusoid_inv_freq(W, cfg.sin_pos_base,
+                                                      device)
         for li, lw in enumerate(self.layers):
             self._name_map.update(lw.named(f"l{li}."))
         self.capture_layers: Optional[List[torch.Tensor]] = None
@@ -551,6 +684,10 @@ class HybridInferenceModel:
         for li, L in enumerate(cfg.layers):
             if L.mixer.kind == "general_delta":
                 shp = shapes.get(f"l{li}.mix.w1")
+                if shp is not None:
+                    L.mixer.decay_rank = int(shp[0])
+            if L.mixer.kind == "gla":
+                shp = shapes.get(f"l{li}.mix.a1")
                 if shp is not None:
                     L.mixer.decay_rank = int(shp[0])
             if L.mixer.kind == "attention" and L.mixer.bias_far > 0:
@@ -633,6 +770,16 @@ class HybridInferenceModel:
                     torch.rand(buf.shape[0], E, generator=g).argsort(1)[
                         :, :buf.shape[1]].int()
                 buf.copy_(t)
+            elif self.prenorm and name.endswith(
+                    ("norm1", "norm2", "final.norm", ".norm")):
+                buf.copy_(1.0 + torch.randn(buf.shape, generator=g) * 0.1)
+            elif self.prenorm and name.endswith("a2.b"):
+                buf.copy_(2.0 + torch.randn(buf.shape, generator=g))
+            elif self.prenorm and (name.endswith(".b")
+                                   or name == "loop.step"):
+                buf.copy_(torch.randn(buf.shape, generator=g) * 0.1)
+            elif name == "bigram":
+                buf.copy_(torch.randn(buf.shape, generator=g) * 0.5)
             elif self.sandwich and name.endswith(
                     ("norm1", "norm2", "norm1b", "norm2b", "final.norm")):
                 buf.copy_(torch.randn(buf.shape, generator=g) * 0.1)
@@ -647,6 +794,9 @@ class HybridInferenceModel:
                 buf.copy_(torch.randn(buf.shape, generator=g) * 0.5)
             elif name.endswith(("canon1", "mix.conv")):
                 buf.copy_(torch.randn(buf.shape, generator=g) * 0.3)
+            elif name == "embed" and self.cfg.embed_scale != 1.0:
+                buf.copy_(torch.randn(buf.shape, generator=g)
+                          / self.cfg.embed_scale)
             elif name in ("embed", "side.embed"):
                 buf.copy_(torch.randn(buf.shape, generator=g))
             else:
@@ -675,6 +825,8 @@ class HybridInferenceModel:
         rows and advances the sequences' recurrent states in place."""
         if self.sandwich:
             return self._forward_sandwich(bt, cache, states)
+        if self.prenorm:
+            return self._forward_prenorm(bt, cache, states)
         cfg, dt = self.cfg, self.dtype
         eps = cfg.norm_eps
         res = self.embed[bt.tokens].float()
@@ -729,6 +881,53 @@ class HybridInferenceModel:
                                                off)
             else:
                 seq.add_scaled_unit_rms(res, y, post, eps, off)
+            if self.capture_layers is not None:
+                self.capture_layers.append(res.clone())
+        return res
+
+    def embed_rows(self, bt: HybridBatch) -> torch.Tensor:
+        """The fp32 embedding output of a packed batch: scaled table row,
+        hashed pair row, sinusoid of the position (each if configured)."""
+        cfg = self.cfg
+        bg = cfg.bigram
+        return seq.embed_compose(
+            self.embed, bt.tokens, cfg.embed_scale, self.pair_embed,
+            bt.prev_tokens, bg.mul_prev if bg else 0, bg.mul_cur if bg else 0,
+            bg.buckets if bg else 0, bt.positions, self.pos_inv_freq)
+
+    def _forward_prenorm(self, bt: HybridBatch, cache, states):
+        """Layer runs of the pre-norm style.  A sublayer's output stays
+        pending until the next norm adds it (times the residual multiplier)
+        to the fp32 stream in the same pass over the row; what a looped
+        span's pass adds at its start (the embedding output again, the
+        pass's vector) joins that pass too."""
+        cfg, dt = self.cfg, self.dtype
+        eps, m, d = cfg.norm_eps, cfg.residual_mult, cfg.token_side_dim
+        starts = cfg.pass_starts()
+        x0 = self.embed_rows(bt)
+        res = x0.clone() if cfg.loop_reinject and starts else x0
+        for ri, li in enumerate(self.runs):
+            L = self.layers[li]
+            rep = starts.get(ri)
+            h = seq.add_rmsnorm_f32res(
+                res, None, L.norm1, eps, dt,
+                extra=x0 if rep and cfg.loop_reinject else None,
+                extra_vec=self.loop_step[rep]
+                if rep is not None and self.loop_step is not None else None)
+            pending = L.mixer.forward(h, bt, ri, self, cache, states)
+            if L.ff is not None:
+                h = seq.add_rmsnorm_f32res(res, pending, L.norm2, eps, dt,
+                                           scale=m)
+                pending = L.ff.forward(h, res, bt)
+            if d > 0:
+                x = seq.residual_add_cast(res, pending, dt, scale=m)
+                gated = seq.gelu_tanh_mul_rows(_mm(x, L.side_gate),
+                                               self.side_embed, bt.tokens,
+                                               li * d)
+                seq.add_scaled_unit_rms(res, _mm(gated, L.side_proj),
+                                        L.side_norm, eps, scale=m)
+            else:
+                seq.residual_add_cast(res, pending, torch.float32, scale=m)
             if self.capture_layers is not None:
                 self.capture_layers.append(res.clone())
         return res
