@@ -412,3 +412,133 @@ def test_gelu_erf(dt):
     x = rnd(33, 70, dt=dt, scale=2.0)
     torch.testing.assert_close(seq.gelu_erf(x.to(DEV)[:, 3:60]).cpu().float(),
                                R.gelu_erf(x[:, 3:60]).float(), **tol(dt))
+
+
+# ------------------ composed embedding, gated linear attention, causal
+# attention with sink and query temperature, clamped gated unit, scaled joins
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("D,pair,pos", [(48, True, True), (37, True, False),
+                                        (200, False, True), (16, False, False)])
+def test_embed_compose(dt, D, pair, pos):
+    V, buckets, N = 50, 23, 19
+    table = rnd(V, D, dt=dt)
+    ptab = rnd(buckets + 1, D, dt=dt) if pair else None
+    tok = torch.randint(0, V, (N,))
+    prev = torch.randint(0, V, (N,))
+    prev[[0, 7, 8]] = -1                     # starts of sequences
+    p = torch.randint(0, 3000, (N,), dtype=torch.int32)
+    f = seq.sinusoid_inv_freq(D, 10000.0, "cpu") if pos else None
+    want = R.embed_compose(table, tok, 3.25, ptab, prev, 31, 7, buckets, p, f)
+    g = lambda t: None if t is None else t.to(DEV)
+    got = seq.embed_compose(g(table), g(tok), 3.25, g(ptab), g(prev), 31, 7,
+                            buckets, g(p), g(f))
+    assert got.dtype == torch.float32
+    torch.testing.assert_close(got.cpu(), want, rtol=1e-5, atol=2e-5)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("H,Dk,Dv,lens", [
+    (3, 32, 32, [6, 1, 3]), (2, 24, 40, [4, 1]), (2, 80, 16, [1, 5]),
+    (1, 128, 70, [3]), (3, 5, 3, [2, 7, 1]), (2, 48, 32, [33, 1])])
+def test_gla_scan(dt, H, Dk, Dv, lens):
+    slots = [2, 0, 3][:len(lens)]
+    bt = batch(lens, slots)
+    N = sum(lens)
+    nk, nv = H * Dk, H * Dv
+    big = rnd(N, 3 * nk + nv + 5, dt=dt)     # operands are column slices
+    cols = lambda t: (t[:, :nk], t[:, nk:2 * nk], t[:, 2 * nk:2 * nk + nv],
+                      t[:, 2 * nk + nv:3 * nk + nv])
+    zb = rnd(nk) + 2.0
+    st0 = rnd(4, H, Dk, Dv, scale=0.3)
+    sc, sg = st0.clone(), st0.clone().to(DEV)
+    want = R.gla_scan(*cols(big), zb, sc, bt["cpu"][0], bt["cpu"][1],
+                      Dk ** -0.5, 1.0 / 3.0)
+    got = seq.gla_scan(*cols(big.to(DEV)), zb.to(DEV), sg, bt[DEV][0],
+                       bt[DEV][1], Dk ** -0.5, 1.0 / 3.0)
+    torch.testing.assert_close(got.cpu(), want, rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(sg.cpu(), sc, rtol=1e-5, atol=1e-5)
+    untouched = [s for s in range(4) if s not in slots]
+    torch.testing.assert_close(sg.cpu()[untouched], st0[untouched], rtol=0,
+                               atol=0)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("groups,gs,shared,act", [
+    (4, 32, True, "silu"), (3, 20, True, "sigmoid"), (6, 70, False, "silu"),
+    (1, 600, True, "silu")])
+def test_group_rmsnorm_gate_forms(dt, groups, gs, shared, act):
+    N, D = 9, groups * gs
+    y = rnd(N, D)
+    w = rnd(gs if shared else D).abs() + 0.5
+    gbig = rnd(N, D + 8, dt=dt)
+    want = R.group_rmsnorm(y, w, groups, 1e-5, dt, gbig[:, 3:3 + D], act)
+    got = seq.group_rmsnorm(y.to(DEV), w.to(DEV), groups, 1e-5, dt,
+                            gbig.to(DEV)[:, 3:3 + D], act)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dt))
+    want = R.group_rmsnorm(y, w, groups, 1e-5, dt)
+    got = seq.group_rmsnorm(y.to(DEV), w.to(DEV), groups, 1e-5, dt)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dt))
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_clamped_glu_and_scaled_joins(dt):
+    N, F = 11, 72
+    gu = rnd(N, 2 * F + 4, dt=dt, scale=2.0)
+    want = R.clamped_glu(gu[:, :F], gu[:, F:2 * F], 1.25, 1.702, 1.0)
+    gd = gu.to(DEV)
+    got = seq.clamped_glu(gd[:, :F], gd[:, F:2 * F], 1.25, 1.702, 1.0)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dt))
+    D = 200
+    res, y, w = rnd(N, D), rnd(N, D, dt=dt), rnd(D).abs() + 0.5
+    ex, exv = rnd(N, D), rnd(D)
+    r0, r1 = res.clone(), res.clone().to(DEV)
+    want = R.add_rmsnorm_f32res(r0, y, w, 1e-6, dt, 0.0, 0.5, ex, exv)
+    got = seq.add_rmsnorm_f32res(r1, y.to(DEV), w.to(DEV), 1e-6, dt, 0.0, 0.5,
+                                 ex.to(DEV), exv.to(DEV))
+    torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dt))
+    torch.testing.assert_close(r1.cpu(), r0, rtol=1e-6, atol=1e-6)
+    got = seq.add_rmsnorm_f32res(r1, None, w.to(DEV), 1e-6, dt,
+                                 extra_vec=exv.to(DEV))
+    want = R.add_rmsnorm_f32res(r0, None, w, 1e-6, dt, extra_vec=exv)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dt))
+    torch.testing.assert_close(r1.cpu(), r0, rtol=1e-6, atol=1e-6)
+    x = seq.residual_add_cast(r1, y.to(DEV), dt, scale=0.3)
+    xw = R.residual_add_cast(r0, y, dt, scale=0.3)
+    torch.testing.assert_close(x.cpu().float(), xw.float(), **tol(dt))
+    seq.add_scaled_unit_rms(r1, y.to(DEV), w.to(DEV), 1e-6, scale=0.7)
+    R.add_scaled_unit_rms(r0, y, w, 1e-6, scale=0.7)
+    torch.testing.assert_close(r1.cpu(), r0, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("H,G,D,Dv,coef,every,lens,starts", [
+    (4, 2, 24, 24, 0.4, 7, [5, 1, 3], [0, 37, 6]),
+    (6, 3, 64, 64, 0.0, 1, [40, 1, 1, 2], [3, 70, 0, 15]),
+    (4, 1, 16, 40, 1.5, 1, [5, 1, 30], [0, 37, 6]),
+    (6, 2, 96, 96, 0.3, 64, [70, 1, 130], [10, 300, 0]),
+    (3, 3, 200, 72, 0.2, 3, [6, 2], [0, 9]),
+    (4, 4, 32, 8, 0.5, 16, [1, 1, 1], [0, 31, 200]),
+])
+def test_causal_attention_with_sink_and_temperature(dt, H, G, D, Dv, coef,
+                                                    every, lens, starts):
+    from polyrl_amd.models.hybrid import UNBOUNDED
+    page = 4
+    cache, ptab, pos, sot, slot = _paged(lens, starts, page, G * (D + Dv), dt)
+    N = sum(lens)
+    q = rnd(N, H * D, dt=dt, scale=2.5)
+    sink = rnd(H, scale=3.0)
+    scale = 1.0 / math.sqrt(D)
+    want = R.gqa_window_attention(q, cache, ptab, sot, pos, H, G, D, Dv,
+                                  UNBOUNDED, 0, None, None, None, scale, dt,
+                                  sink, coef, every)
+    plain = R.gqa_window_attention(q, cache, ptab, sot, pos, H, G, D, Dv,
+                                   UNBOUNDED, 0, None, None, None, scale, dt)
+    assert float((want.float() - plain.float()).abs().max()) > 0.05
+    g = lambda t: t.to(DEV)
+    tiles = seq.attention_tiles(lens, DEV)
+    for tl in (None, tiles):                 # one wave per row; matrix cores
+        got = seq.gqa_window_attention(
+            g(q), g(cache), g(ptab), g(sot), g(pos), H, G, D, Dv, UNBOUNDED,
+            0, None, None, None, scale, dt, tiles=tl, sink=g(sink),
+            q_temp_coef=coef, q_temp_every=every)
+        torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dt))
