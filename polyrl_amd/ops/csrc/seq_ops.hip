@@ -19,8 +19,8 @@
 // mode 0: res += ys*y [+ ex] [+ exv]; out = res * rsqrt(mean(res^2)+eps) * g
 // mode 1: res += ys*y; out = res (cast)                          (no norm)
 // mode 2: res += ys * y * rsqrt(mean(y^2)+eps) * g               (out unused)
-// mode 3: mode 2, then out = res * rsqrt(mean(res^2)+eps) * (off + w2)
-//         (the joint between two normed sublayers in one pass)
+// mode 3: mode 2 [+ ex] [+ exv], then out = res * rsqrt(mean(res^2)+eps)
+//         * (off + w2)  (the joint between two normed sublayers in one pass)
 // ys scales the branch that joins the stream; ex (rows, D) fp32 and exv (D)
 // fp32 are what a pass of a looped span adds at its start.
 template <typename T>
@@ -65,9 +65,11 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(
     return;
   }
   float ss2 = 0.f;
+  const float* er3 = ex ? ex + row * D : nullptr;
   for (int i = threadIdx.x; i < D; i += 256) {
-    const float f =
-        rr[i] + ys * (ldf(yr + i) * inv * (w[wn == 1 ? 0 : i] + off));
+    float f = rr[i] + ys * (ldf(yr + i) * inv * (w[wn == 1 ? 0 : i] + off));
+    if (er3) f += er3[i];
+    if (exv) f += exv[i];
     rr[i] = f;
     ss2 += f * f;
   }
@@ -113,12 +115,14 @@ void seq_add_rmsnorm(torch::Tensor out, torch::Tensor res, torch::Tensor y,
   const float* exv = nullptr;
   if (extra.defined() && extra.numel() > 0) {
     CHECK_F32(extra);
-    TORCH_CHECK(mode == 0 && extra.numel() == res.numel(), "extra shape");
+    TORCH_CHECK((mode == 0 || mode == 3) && extra.numel() == res.numel(),
+                "extra shape");
     ex = extra.data_ptr<float>();
   }
   if (extra_vec.defined() && extra_vec.numel() > 0) {
     CHECK_F32(extra_vec);
-    TORCH_CHECK(mode == 0 && extra_vec.numel() == D, "extra_vec shape");
+    TORCH_CHECK((mode == 0 || mode == 3) && extra_vec.numel() == D,
+                "extra_vec shape");
     exv = extra_vec.data_ptr<float>();
   }
   const bool out_is_res = out.data_ptr() == res.data_ptr();

@@ -17,10 +17,10 @@
 // Per-token inputs of a lane's rows are contiguous and come in with 16-byte
 // loads when the layout allows (scalar loads otherwise); the inputs of token
 // t+1 are requested before the arithmetic of token t.  The delta rule's
-// decay and removal rate cost three exponentials per row (gated linear
-// attention's decay an exponential and a logarithm): the 16 column
+// decay and removal rate cost three exponentials per row: the 16 column
 // lanes of a row group would all compute the same ones, so each computes
-// one sixteenth and the group exchanges them by lane shuffles.
+// one sixteenth and the group exchanges them by lane shuffles.  Gated
+// linear attention stages whole tiles of tokens in LDS instead (below).
 // All state math is fp32 for bf16 or fp32 inputs.
 #include <torch/extension.h>
 #include <ATen/hip/HIPContext.h>
@@ -239,28 +239,29 @@ void seq_delta_rule(torch::Tensor out, torch::Tensor r, torch::Tensor k,
 // ------------------------------------------------- gated linear attention
 // decay of key channel i: sigmoid(z_i + zb_i)^(1/tau)
 //   = exp(inv_tau * log_sigmoid(z_i + zb_i)), fp32
-template <int RPL>
-struct GlaIn {
-  static constexpr int NC = (RPL + 15) / 16;   // rows whose decay I compute
-  float q[RPL], k[RPL];
-  float zl[NC];
-  float v;
-};
+//
+// Same lane mapping as above, but the token inputs do not come to the lanes
+// one token at a time (a dependent global load per token is what bounds a
+// long portion): the block stages TT tokens at once in LDS -- scaled queries,
+// keys and the decays, each computed once per (token, channel) instead of
+// once per column block -- and the waves then walk the tile out of LDS, where
+// the 16 column lanes of a row group read the same words (broadcast).  A
+// thread's words of the next tile are requested into registers before the
+// current tile is walked.
+// sum over the four lanes 4j .. 4j+3 (the row groups of one column) by two
+// quad permutes in the VALU data path: partner lane^2, then lane^1
+DEV_INLINE float quad_sum(float x) {
+  x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+      0, __builtin_bit_cast(int, x), 0x4E, 0xF, 0xF, false));  // [2,3,0,1]
+  x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+      0, __builtin_bit_cast(int, x), 0xB1, 0xF, 0xF, false));  // [1,0,3,2]
+  return x;
+}
 
-template <typename T, int RPL>
-DEV_INLINE void gla_load(GlaIn<RPL>& in, const T* q, const T* k, const T* v,
-                         const T* zl, long ldq, long ldk, long ldv, long ldz,
-                         long n, int hoff_k, int row0, int Dk, int vcol,
-                         bool colok, int ci, bool vec) {
-  load_rows<T, RPL>(in.q, q + n * ldq + hoff_k + row0, row0, Dk, vec);
-  load_rows<T, RPL>(in.k, k + n * ldk + hoff_k + row0, row0, Dk, vec);
-#pragma unroll
-  for (int c = 0; c < GlaIn<RPL>::NC; ++c) {
-    const int i = ci + 16 * c;
-    const bool ok = i < RPL && row0 + i < Dk;
-    in.zl[c] = ok ? ldf(zl + n * ldz + hoff_k + row0 + i) : 0.f;
-  }
-  in.v = colok ? ldf(v + n * ldv + vcol) : 0.f;
+// tokens per LDS tile: at most 32, and the tile within 48 KB
+constexpr int gla_tile_tokens(int dkp) {
+  const int fit = 48 * 1024 / (4 * (3 * dkp + 64));
+  return fit < 32 ? fit : 32;
 }
 
 template <typename T, int RPL>
@@ -270,8 +271,15 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(
     const T* __restrict__ zl, long ldq, long ldk, long ldv, long ldz,
     const float* __restrict__ z_bias, float* __restrict__ state,
     const int* __restrict__ cu_q, const int* __restrict__ state_slot, int H,
-    int Dk, int Dv, float q_scale, float inv_tau, bool vec) {
-  constexpr int NC = GlaIn<RPL>::NC;
+    int Dk, int Dv, float q_scale, float inv_tau) {
+  constexpr int DKP = RG * RPL;         // key rows incl. padding
+  constexpr int TT = gla_tile_tokens(DKP);
+  constexpr int NIT = (TT * DKP + 255) / 256;   // staged words per thread
+  constexpr int NVI = (TT * 64 + 255) / 256;
+  __shared__ __attribute__((aligned(16))) float q_s[TT * DKP];  // * q_scale
+  __shared__ __attribute__((aligned(16))) float k_s[TT * DKP];
+  __shared__ __attribute__((aligned(16))) float d_s[TT * DKP];  // decays
+  __shared__ float v_s[TT * 64];        // this block's columns
   const int cblocks = (Dv + 63) / 64;
   const int b = blockIdx.x / (H * cblocks);
   const int h = (blockIdx.x / cblocks) % H;
@@ -284,49 +292,87 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(
   const int row0 = rg * RPL;
   const bool colok = col < Dv;
   const int q0 = cu_q[b], q1 = cu_q[b + 1];
-  if (q1 <= q0) return;
-  // a whole wave past the last column has nothing to do (wave-uniform)
-  if (cb * 64 + wid * COLS_PER_WAVE >= Dv) return;
+  if (q1 <= q0) return;                           // the whole block
+  // a wave past the last column only helps to stage the tiles
+  const bool wave_live = cb * 64 + wid * COLS_PER_WAVE < Dv;
 
   float* S = state + (((long)state_slot[b] * H + h) * Dk) * Dv;
-  float s[RPL], zbc[NC];
+  float s[RPL];
 #pragma unroll
   for (int i = 0; i < RPL; ++i) {
     const int row = row0 + i;
     s[i] = (colok && row < Dk) ? S[(long)row * Dv + col] : 0.f;
   }
-#pragma unroll
-  for (int c = 0; c < NC; ++c) {
-    const int i = ci + 16 * c;
-    const bool ok = i < RPL && row0 + i < Dk;
-    zbc[c] = ok ? z_bias[h * Dk + row0 + i] : 0.f;
-  }
   const int hoff_k = h * Dk;
   const int vcol = h * Dv + col;
 
-  GlaIn<RPL> cur, nxt;
-  gla_load<T, RPL>(cur, q, k, v, zl, ldq, ldk, ldv, ldz, q0, hoff_k, row0, Dk,
-                   vcol, colok, ci, vec);
-  for (int n = q0; n < q1; ++n) {
-    if (n + 1 < q1)
-      gla_load<T, RPL>(nxt, q, k, v, zl, ldq, ldk, ldv, ldz, n + 1, hoff_k,
-                       row0, Dk, vcol, colok, ci, vec);
-    // my share of the decays: rows ci, ci+16, .. of this row group
-    float decm[NC];
+  // a tile's words of this thread, requested one tile ahead of their use
+  float rq[NIT], rk[NIT], rz[NIT], rv[NVI];
+  auto fetch = [&](int n0) {
+    const int cnt = q1 - n0 < TT ? q1 - n0 : TT;
 #pragma unroll
-    for (int c = 0; c < NC; ++c)
-      decm[c] = expf(-inv_tau * softplusf_acc(-(cur.zl[c] + zbc[c])));
-    float o = 0.f;
-#pragma unroll
-    for (int i = 0; i < RPL; ++i) {
-      const int src = (i % 16) * RG + rg;          // lane that owns row i
-      const float dec = __shfl(decm[i / 16], src, WAVE_SIZE);
-      s[i] = dec * s[i] + cur.k[i] * cur.v;
-      o += s[i] * (cur.q[i] * q_scale);
+    for (int it = 0; it < NIT; ++it) {
+      if (it * 256 >= cnt * DKP) break;         // block-uniform
+      const int idx = threadIdx.x + it * 256;
+      const int t = idx / DKP, r = idx % DKP;
+      const bool ok = t < cnt && r < Dk;
+      const long n = n0 + t;
+      rq[it] = ok ? ldf(q + n * ldq + hoff_k + r) : 0.f;
+      rk[it] = ok ? ldf(k + n * ldk + hoff_k + r) : 0.f;
+      rz[it] = ok ? ldf(zl + n * ldz + hoff_k + r) + z_bias[hoff_k + r]
+                  : INFINITY;
     }
-    o = lanegroup_sum<RG>(o);
-    if (colok && rg == 0) out[(long)n * H * Dv + vcol] = o;
-    cur = nxt;
+#pragma unroll
+    for (int it = 0; it < NVI; ++it) {
+      if (it * 256 >= cnt * 64) break;
+      const int idx = threadIdx.x + it * 256;
+      const int t = idx >> 6, c = cb * 64 + (idx & 63);
+      rv[it] = (t < cnt && c < Dv)
+                   ? ldf(v + (long)(n0 + t) * ldv + h * Dv + c) : 0.f;
+    }
+  };
+  fetch(q0);
+  for (int n0 = q0; n0 < q1; n0 += TT) {
+    const int cnt = q1 - n0 < TT ? q1 - n0 : TT;
+    __syncthreads();                    // the tile before this one is used up
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+      const int idx = threadIdx.x + it * 256;
+      if (idx < cnt * DKP) {
+        q_s[idx] = rq[it] * q_scale;
+        k_s[idx] = rk[it];
+        d_s[idx] = expf(-inv_tau * softplusf_acc(-rz[it]));
+      }
+    }
+#pragma unroll
+    for (int it = 0; it < NVI; ++it) {
+      const int idx = threadIdx.x + it * 256;
+      if (idx < cnt * 64) v_s[idx] = rv[it];
+    }
+    __syncthreads();
+    if (n0 + TT < q1) fetch(n0 + TT);   // in flight while this tile is walked
+    if (!wave_live) continue;
+    static_assert(RG == 4, "quad_sum adds the four row groups");
+    auto step = [&](int t) {
+      const float* qr = q_s + t * DKP + row0;
+      const float* kr = k_s + t * DKP + row0;
+      const float* dr = d_s + t * DKP + row0;
+      const float vv = v_s[t * 64 + wid * COLS_PER_WAVE + ci];
+      float o = 0.f;
+#pragma unroll
+      for (int i = 0; i < RPL; ++i) {
+        s[i] = dr[i] * s[i] + kr[i] * vv;
+        o += s[i] * qr[i];
+      }
+      o = quad_sum(o);
+      if (colok && rg == 0) out[(long)(n0 + t) * H * Dv + vcol] = o;
+    };
+    int t = 0;
+    for (; t + 4 <= cnt; t += 4) {      // four tokens' LDS reads in flight
+#pragma unroll
+      for (int u = 0; u < 4; ++u) step(t + u);
+    }
+    for (; t < cnt; ++t) step(t);
   }
 #pragma unroll
   for (int i = 0; i < RPL; ++i) {
@@ -342,9 +388,7 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(
       (const T*)z_lin.data_ptr(), q.stride(0), k.stride(0), v.stride(0),     \
       z_lin.stride(0), z_bias.data_ptr<float>(), state.data_ptr<float>(),    \
       cu_q.data_ptr<int>(), state_slot.data_ptr<int>(), H, Dk, Dv,           \
-      (float)q_scale, (float)inv_tau,                                        \
-      rows_vectorizable<T>(q, 0, Dk, RPLV) &&                                \
-          rows_vectorizable<T>(k, 0, Dk, RPLV))
+      (float)q_scale, (float)inv_tau)
 
 void seq_gla_scan(torch::Tensor out, torch::Tensor q, torch::Tensor k,
                   torch::Tensor v, torch::Tensor z_lin, torch::Tensor z_bias,

@@ -129,18 +129,23 @@ def embed_compose(table, tokens, scale: float, pair_table, prev_tokens,
 def add_unit_rms_then_norm(res: torch.Tensor, y: torch.Tensor,
                            w_post: torch.Tensor, w_next: torch.Tensor,
                            eps: float, out_dtype: torch.dtype,
-                           offset: float = 0.0) -> torch.Tensor:
+                           offset: float = 0.0, scale: float = 1.0,
+                           extra: Optional[torch.Tensor] = None,
+                           extra_vec: Optional[torch.Tensor] = None
+                           ) -> torch.Tensor:
     """The joint between two normed sublayers in one pass over the row:
-    res += y / rms(y) * (offset + w_post) in place, then returns
+    res += scale * y / rms(y) * (offset + w_post) [+ extra (N, D) fp32]
+    [+ extra_vec (D,) fp32] in place, then returns
     res / rms(res) * (offset + w_next) as out_dtype."""
     if res.is_cuda:
         out = torch.empty(res.shape, dtype=out_dtype, device=res.device)
         e = torch.Tensor()
         _ext().seq_add_rmsnorm(out, res, y, w_post, eps, 3, offset, w_next,
-                               1.0, e, e)
+                               scale, extra if extra is not None else e,
+                               extra_vec if extra_vec is not None else e)
         return out
     return R.add_unit_rms_then_norm(res, y, w_post, w_next, eps, out_dtype,
-                                    offset)
+                                    offset, scale, extra, extra_vec)
 
 
 def causal_conv_state(x, w, bias, state, cu_q, state_slot, seq_of_tok,

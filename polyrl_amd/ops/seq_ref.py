@@ -41,9 +41,11 @@ def add_scaled_unit_rms(res, y, weight, eps, offset=0.0, scale=1.0):
     res.add_(add * scale if scale != 1.0 else add)
 
 
-def add_unit_rms_then_norm(res, y, w_post, w_next, eps, out_dtype, offset):
-    add_scaled_unit_rms(res, y, w_post, eps, offset)
-    return add_rmsnorm_f32res(res, None, w_next, eps, out_dtype, offset)
+def add_unit_rms_then_norm(res, y, w_post, w_next, eps, out_dtype, offset,
+                           scale=1.0, extra=None, extra_vec=None):
+    add_scaled_unit_rms(res, y, w_post, eps, offset, scale)
+    return add_rmsnorm_f32res(res, None, w_next, eps, out_dtype, offset,
+                              extra=extra, extra_vec=extra_vec)
 
 
 def causal_conv_state(x, w, bias, state, cu_q, state_slot, seq_of_tok,

@@ -896,24 +896,42 @@ class HybridInferenceModel:
             bg.buckets if bg else 0, bt.positions, self.pos_inv_freq)
 
     def _forward_prenorm(self, bt: HybridBatch, cache, states):
-        """Layer runs of the pre-norm style.  A sublayer's output stays
-        pending until the next norm adds it (times the residual multiplier)
-        to the fp32 stream in the same pass over the row; what a looped
-        span's pass adds at its start (the embedding output again, the
-        pass's vector) joins that pass too."""
+        """Layer runs of the pre-norm style.  What a sublayer or the
+        token-side input adds to the fp32 stream (times the residual
+        multiplier) stays pending until the next norm, which adds it in the
+        same pass over the row; what a looped span's pass adds at its start
+        (the embedding output again, the pass's vector) joins that pass
+        too."""
         cfg, dt = self.cfg, self.dtype
         eps, m, d = cfg.norm_eps, cfg.residual_mult, cfg.token_side_dim
         starts = cfg.pass_starts()
         x0 = self.embed_rows(bt)
-        res = x0.clone() if cfg.loop_reinject and starts else x0
+        res = x0.clone() if cfg.loop_reinject and len(starts) > 1 else x0
+        pending = side = None     # sublayer output / (side output, weight)
+
+        def settle():
+            nonlocal pending, side
+            if side is not None:
+                seq.add_scaled_unit_rms(res, side[0], side[1], eps, scale=m)
+            elif pending is not None:
+                seq.residual_add_cast(res, pending, torch.float32, scale=m)
+            pending = side = None
+
         for ri, li in enumerate(self.runs):
             L = self.layers[li]
             rep = starts.get(ri)
-            h = seq.add_rmsnorm_f32res(
-                res, None, L.norm1, eps, dt,
-                extra=x0 if rep and cfg.loop_reinject else None,
-                extra_vec=self.loop_step[rep]
-                if rep is not None and self.loop_step is not None else None)
+            extra = x0 if rep and cfg.loop_reinject else None
+            vec = self.loop_step[rep] \
+                if rep is not None and self.loop_step is not None else None
+            if side is not None:
+                h = seq.add_unit_rms_then_norm(res, side[0], side[1], L.norm1,
+                                               eps, dt, scale=m, extra=extra,
+                                               extra_vec=vec)
+            else:
+                h = seq.add_rmsnorm_f32res(res, pending, L.norm1, eps, dt,
+                                           scale=m, extra=extra,
+                                           extra_vec=vec)
+            side = None
             pending = L.mixer.forward(h, bt, ri, self, cache, states)
             if L.ff is not None:
                 h = seq.add_rmsnorm_f32res(res, pending, L.norm2, eps, dt,
@@ -921,15 +939,15 @@ class HybridInferenceModel:
                 pending = L.ff.forward(h, res, bt)
             if d > 0:
                 x = seq.residual_add_cast(res, pending, dt, scale=m)
+                pending = None
                 gated = seq.gelu_tanh_mul_rows(_mm(x, L.side_gate),
                                                self.side_embed, bt.tokens,
                                                li * d)
-                seq.add_scaled_unit_rms(res, _mm(gated, L.side_proj),
-                                        L.side_norm, eps, scale=m)
-            else:
-                seq.residual_add_cast(res, pending, torch.float32, scale=m)
+                side = (_mm(gated, L.side_proj), L.side_norm)
             if self.capture_layers is not None:
+                settle()
                 self.capture_layers.append(res.clone())
+        settle()
         return res
 
     @torch.no_grad()

@@ -439,7 +439,8 @@ def test_embed_compose(dt, D, pair, pos):
 @pytest.mark.parametrize("dt", DTYPES)
 @pytest.mark.parametrize("H,Dk,Dv,lens", [
     (3, 32, 32, [6, 1, 3]), (2, 24, 40, [4, 1]), (2, 80, 16, [1, 5]),
-    (1, 128, 70, [3]), (3, 5, 3, [2, 7, 1]), (2, 48, 32, [33, 1])])
+    (1, 128, 70, [3]), (3, 5, 3, [2, 7, 1]), (2, 48, 32, [33, 1]),
+    (2, 64, 128, [70, 1, 32]), (1, 200, 16, [40, 15]), (1, 256, 8, [29])])
 def test_gla_scan(dt, H, Dk, Dv, lens):
     slots = [2, 0, 3][:len(lens)]
     bt = batch(lens, slots)
@@ -508,6 +509,15 @@ def test_clamped_glu_and_scaled_joins(dt):
     seq.add_scaled_unit_rms(r1, y.to(DEV), w.to(DEV), 1e-6, scale=0.7)
     R.add_scaled_unit_rms(r0, y, w, 1e-6, scale=0.7)
     torch.testing.assert_close(r1.cpu(), r0, rtol=1e-5, atol=1e-5)
+    w2 = rnd(D).abs() + 0.5
+    for e1, e2 in ((ex, exv), (None, exv), (None, None)):
+        gd = lambda t: None if t is None else t.to(DEV)
+        got = seq.add_unit_rms_then_norm(r1, y.to(DEV), w.to(DEV), w2.to(DEV),
+                                         1e-6, dt, 0.0, 0.4, gd(e1), gd(e2))
+        want = R.add_unit_rms_then_norm(r0, y, w, w2, 1e-6, dt, 0.0, 0.4, e1,
+                                        e2)
+        torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dt))
+        torch.testing.assert_close(r1.cpu(), r0, rtol=1e-5, atol=1e-5)
 
 
 @pytest.mark.parametrize("dt", DTYPES)
