@@ -132,7 +132,7 @@ class WindowAttnSpec:
     the bucket of distance n is n below half the table's rows, logarithmic
     steps up to ``bias_far`` above), biases on the query / key / value
     projections (``qkv_bias``), one learned logit per head that joins the
-    softmax denominator without a key or a value (``sink``), and a query
+    softmax denominator and contributes no value row (``sink``), and a query
     temperature ``1 + q_temp_coef * ln(floor((p + 1) / q_temp_every) + 1)``
     at position p.  ``window = UNBOUNDED`` is plain causal attention."""
     heads: int
@@ -229,8 +229,8 @@ class HybridConfig:
     norm_offset: float = 0.0
     residual_mult: float = 1.0
     # the embedding: table row * embed_scale [+ hashed pair row]
-    # [+ sinusoid of the position: entry 2i = sin(p * base^(-2i/width)),
-    # entry 2i+1 = cos of the same angle; 0 = none]
+    # [+ sinusoid of the position p: angles p * base^(-2i/width), sines at
+    # the even entries, cosines at the odd ones; 0 = none]
     embed_scale: float = 1.0
     bigram: Optional[BigramSpec] = None
     sin_pos_base: float = 0.0

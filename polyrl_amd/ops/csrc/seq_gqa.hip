@@ -17,10 +17,11 @@
 // ranges [0, min(keep, lo)) and [lo, p] are walked as one list.  Scores, the
 // optional distance-bucket bias rel[bucket[p-j], head], the online softmax
 // and the per-head sigmoid gate are fp32.  Two further options: a sink, one
-// learned logit per head that joins the softmax denominator once without a
-// key or a value (the running maximum starts at the sink, the running sum at
-// one), and a query temperature that multiplies the score scale of the row at
-// position p by 1 + coef * ln(floor((p + 1) / every) + 1).
+// learned logit per head that is one more term of the softmax denominator
+// and adds nothing to the weighted sum (the running maximum starts at the
+// sink, the running sum at one), and a query temperature that multiplies
+// the score scale of the row at position p by
+// 1 + coef * ln(floor((p + 1) / every) + 1).
 #include <torch/extension.h>
 #include <ATen/hip/HIPContext.h>
 

@@ -148,8 +148,8 @@ void seq_add_rmsnorm(torch::Tensor out, torch::Tensor res, torch::Tensor y,
 // ------------------------------------------------------ composed embedding
 // out[n] = table[tok] * scale [+ pair[row]] [+ sinusoid(pos)], fp32.
 // row = (prev * mul_prev + tok * mul_cur) mod buckets, or ``buckets`` (the
-// table's last row) where prev < 0.  Sinusoid: entry 2i = sin(a), entry
-// 2i+1 = cos(a), a = fp32(pos) * inv_freq[i].
+// table's last row) where prev < 0.  Sinusoid: sin(a_i) at the even entry
+// 2i and cos(a_i) at the odd one, a_i = fp32(pos) * inv_freq[i].
 template <typename T>
 __global__ __launch_bounds__(256) void embed_compose_kernel(
     float* __restrict__ out, const T* __restrict__ table,

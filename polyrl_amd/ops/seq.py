@@ -108,8 +108,8 @@ def embed_compose(table, tokens, scale: float, pair_table, prev_tokens,
     """The fp32 embedding output (N, D): table[token] * scale
     [+ pair_table[(prev * mul_prev + token * mul_cur) mod buckets], row
     ``buckets`` where prev < 0 (a sequence's first token)]
-    [+ the sinusoid of the position: entry 2i = sin(fp32(p) * inv_freq[i]),
-    entry 2i+1 = cos of the same angle]."""
+    [+ the sinusoid of the position: with angles a_i = fp32(p) * inv_freq[i],
+    sines sit at the even entries (2i) and cosines at the odd ones]."""
     if table.is_cuda:
         out = torch.empty(tokens.shape[0], table.shape[1],
                           dtype=torch.float32, device=table.device)

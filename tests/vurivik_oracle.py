@@ -53,7 +53,8 @@ def bigram_row(prev, cur, bg):
 
 
 def sinusoid(p, width):
-    """Entry 2i = sin(p * 10000^(-2i/width)), entry 2i+1 = cos of it."""
+    """Position vector: angles a_i = p / 10000^(2i/width); sines at the
+    even places, cosines at the odd ones."""
     out = torch.zeros(width, dtype=DT)
     for i in range((width + 1) // 2):
         ang = p * 10000.0 ** (-2.0 * i / width)
@@ -112,8 +113,9 @@ def query_temperature(p, qt):
 
 
 def attention_mixer(hs, W, p, m):
-    """Causal grouped-query softmax attention; the denominator also holds
-    exp(sink_h), which has no key and no value."""
+    """Causal grouped-query softmax attention with one extra term
+    exp(sink_h) in every head's denominator (nothing is added to the
+    weighted sum for it)."""
     H, G = int(m["heads"]), int(m["kv_heads"])
     D, Dv = int(m["dim"]), int(m["vdim"])
     T = hs.shape[0]
