@@ -2,7 +2,7 @@
 //
 // Same operation as gqa_attn_kernel (seq_gqa.hip), which stays the fp32 /
 // odd-size / single-token path.  A block is 4 waves x 16 rows: up to 64
-// consecutive tokens of one sequence for query head blockIdx.y.  Their
+// consecutive tokens of one sequence for one query head.  Their
 // windows overlap, so the block walks the union of the visible keys in tiles
 // of 32 -- first the kept first tokens that lie before the union's window
 // ([0, min(keep, kmin))), then [kmin, last position] -- and masks per
@@ -17,6 +17,12 @@
 // The next tiles are fetched into registers while the current ones are
 // multiplied.
 // K-tile bytes are XOR-swizzled by row inside each 64-byte chunk.
+//
+// Grid: one dimension.  Workgroups go to the 8 XCDs in turn (id mod 8), each
+// with an L2 of its own, so the id is taken apart as XCD = id % 8 and, inside
+// an XCD's sequence, the H/G query heads that share a key/value head follow
+// each other for the same row tile: their K and V tiles are fetched into that
+// XCD's L2 once and hit there for the other heads of the group.
 #include <torch/extension.h>
 #include <ATen/hip/HIPContext.h>
 
@@ -28,6 +34,7 @@ typedef __attribute__((ext_vector_type(4))) int i32x4_t;
 
 constexpr int GKV = 32;          // keys per tile
 constexpr int GQA_MAX_REL = 256; // bias-table rows held in LDS
+constexpr int GQA_XCDS = 8;      // accelerator dies, each with its own L2
 
 template <int KS>
 DEV_INLINE int gtile_off(int row, int byte_col) {
@@ -42,7 +49,7 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(
     const int* __restrict__ page_table, int max_pages,
     const int* __restrict__ seq_of_tok, const int* __restrict__ positions,
     const int* __restrict__ tile_n0, const int* __restrict__ tile_cnt,
-    const float* __restrict__ rel, int rel_rows,
+    int ntiles_rows, const float* __restrict__ rel, int rel_rows,
     const int* __restrict__ dist_bucket,
     const bf16_t* __restrict__ gate, long ldg, int H, int G, int D, int Dv,
     int page_size, int window, int keep, float scale,
@@ -57,12 +64,20 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(
   const int lane = threadIdx.x & 63;
   const int wid = threadIdx.x >> 6;
   const int l15 = lane & 15, lhi = lane >> 4;
-  const int h = blockIdx.y;
-  const int g = h / (H / G);
+  const int per = H / G;                 // query heads per key/value head
+  const int xcd = blockIdx.x % GQA_XCDS;
+  const int seq_in_xcd = blockIdx.x / GQA_XCDS;
+  const int unit = (seq_in_xcd / per) * GQA_XCDS + xcd;   // (tile, kv head)
+  if (unit >= ntiles_rows * G) return;   // padding of the last round
+  // later row tiles see more keys: they start first, the short ones fill
+  // the end of the launch
+  const int tile = ntiles_rows - 1 - unit % ntiles_rows;
+  const int g = unit / ntiles_rows;
+  const int h = g * per + seq_in_xcd % per;
   const int row = G * (D + Dv);
   const int koff = g * D, voff = G * D + g * Dv;
-  const int n0 = tile_n0[blockIdx.x];
-  const int cnt = tile_cnt[blockIdx.x];
+  const int n0 = tile_n0[tile];
+  const int cnt = tile_cnt[tile];
   const int b = seq_of_tok[n0];
   const int* ptab = page_table + (long)b * max_pages;
   const int pos0 = positions[n0];
@@ -273,7 +288,8 @@ void seq_gqa_window_attention(torch::Tensor out, torch::Tensor q,
       (const bf16_t*)cache.data_ptr(), page_table.data_ptr<int>(),            \
       (int)page_table.size(1), seq_of_tok.data_ptr<int>(),                    \
       positions.data_ptr<int>(), tile_n0.data_ptr<int>(),                     \
-      tile_cnt.data_ptr<int>(), has_rel ? rel.data_ptr<float>() : nullptr,    \
+      tile_cnt.data_ptr<int>(), ntiles,                                       \
+      has_rel ? rel.data_ptr<float>() : nullptr,                              \
       has_rel ? (int)rel.size(0) : 0,                                         \
       has_rel ? dist_bucket.data_ptr<int>() : nullptr,                        \
       has_gate ? (const bf16_t*)gate.data_ptr() : nullptr,                    \
@@ -309,7 +325,11 @@ void seq_gqa_window_attention_mfma(
   }
   const int ntiles = tile_n0.numel();
   if (q.size(0) == 0 || ntiles == 0) return;
-  const dim3 grid(ntiles, H);
+  // (tile, kv head) units in rounds of one per XCD, H/G heads per unit
+  const long units = (long)ntiles * G;
+  const long rounds = (units + GQA_XCDS - 1) / GQA_XCDS;
+  TORCH_CHECK(rounds * GQA_XCDS * (H / G) < (1L << 31), "grid too large");
+  const dim3 grid((unsigned)(rounds * GQA_XCDS * (H / G)));
   auto stream = at::hip::getCurrentHIPStream();
   switch (ks) {
     case 1: GQA_MFMA_LAUNCH(1); break;
