@@ -409,7 +409,7 @@ void seq_gla_scan(torch::Tensor out, torch::Tensor q, torch::Tensor k,
   auto dt = q.scalar_type();
   TORCH_CHECK(k.scalar_type() == dt && v.scalar_type() == dt &&
               z_lin.scalar_type() == dt);
-  TORCH_CHECK(Dk <= 256, "gated linear attention: key dim above 256 not supported");
+  TORCH_CHECK(Dk <= 512, "gated linear attention: key dim above 512 not supported");
   const int B = state_slot.numel();
   TORCH_CHECK(cu_q.numel() == B + 1);
   if (N == 0 || B == 0) return;
@@ -421,7 +421,8 @@ void seq_gla_scan(torch::Tensor out, torch::Tensor q, torch::Tensor k,
     else if (rpl <= 8) GLA_LAUNCH(8);
     else if (rpl <= 16) GLA_LAUNCH(16);
     else if (rpl <= 32) GLA_LAUNCH(32);
-    else GLA_LAUNCH(64);
+    else if (rpl <= 64) GLA_LAUNCH(64);
+    else GLA_LAUNCH(128);
   });
   HIP_CHECK_KERNEL();
 }

@@ -800,7 +800,9 @@ class Engine:
             n = len(toks)
             # the token before each row: the request's own history for the
             # portion's first row (-1 at the start of the sequence)
-            if start == 0:
+            if n == 0:
+                pass
+            elif start == 0:
                 prev.append(-1)
             elif start - 1 < len(r.input_ids):
                 prev.append(r.input_ids[start - 1])

@@ -440,7 +440,8 @@ def test_embed_compose(dt, D, pair, pos):
 @pytest.mark.parametrize("H,Dk,Dv,lens", [
     (3, 32, 32, [6, 1, 3]), (2, 24, 40, [4, 1]), (2, 80, 16, [1, 5]),
     (1, 128, 70, [3]), (3, 5, 3, [2, 7, 1]), (2, 48, 32, [33, 1]),
-    (2, 64, 128, [70, 1, 32]), (1, 200, 16, [40, 15]), (1, 256, 8, [29])])
+    (2, 64, 128, [70, 1, 32]), (1, 200, 16, [40, 15]), (1, 256, 8, [29]),
+    (1, 320, 24, [11, 2])])
 def test_gla_scan(dt, H, Dk, Dv, lens):
     slots = [2, 0, 3][:len(lens)]
     bt = batch(lens, slots)
