@@ -685,7 +685,7 @@ def vurivik_preset(width: int, layers: int, vocab: int = 32000,
     for li in range(layers):
         if gla_every and li % gla_every == gla_every - 1:
             out.append(HybridLayerSpec(
-                GLASpec(heads=gh, dim=hd, vdim=2 * hd, tau=16.0,
+                GLASpec(heads=gh, dim=hd, vdim=2 * hd, tau=8.0,
                         decay_rank=16), None))
         else:
             out.append(HybridLayerSpec(
@@ -698,9 +698,9 @@ def vurivik_preset(width: int, layers: int, vocab: int = 32000,
     return HybridConfig(
         arch="vurivik", vocab_size=vocab, hidden_size=width, layers=out,
         norm_eps=1e-5, canon_taps=1, token_side_dim=max(8, width // 16),
-        layer_style="prenorm", residual_mult=0.5,
-        embed_scale=math.sqrt(width),
-        bigram=BigramSpec(buckets=65521, mul_prev=31, mul_cur=7),
+        layer_style="prenorm", residual_mult=0.6,
+        embed_scale=8.0,
+        bigram=BigramSpec(buckets=65521, mul_prev=257, mul_cur=13),
         sin_pos_base=10000.0, loop=loop, loop_reinject=bool(loop),
         loop_step=bool(loop)).validate()
 

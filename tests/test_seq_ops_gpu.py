@@ -428,9 +428,9 @@ def test_embed_compose(dt, D, pair, pos):
     prev[[0, 7, 8]] = -1                     # starts of sequences
     p = torch.randint(0, 3000, (N,), dtype=torch.int32)
     f = seq.sinusoid_inv_freq(D, 10000.0, "cpu") if pos else None
-    want = R.embed_compose(table, tok, 3.25, ptab, prev, 31, 7, buckets, p, f)
+    want = R.embed_compose(table, tok, 3.25, ptab, prev, 29, 3, buckets, p, f)
     g = lambda t: None if t is None else t.to(DEV)
-    got = seq.embed_compose(g(table), g(tok), 3.25, g(ptab), g(prev), 31, 7,
+    got = seq.embed_compose(g(table), g(tok), 3.25, g(ptab), g(prev), 29, 3,
                             buckets, g(p), g(f))
     assert got.dtype == torch.float32
     torch.testing.assert_close(got.cpu(), want, rtol=1e-5, atol=2e-5)
