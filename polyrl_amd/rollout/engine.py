@@ -472,6 +472,14 @@ class Engine:
         self.enable_hip_graphs = False
         self._graphs, self._graph_pool = {}, None
         self._decode_buckets = False
+        # pure decode steps of a model whose forward takes no decision on
+        # the host replay one captured hipGraph per batch size instead of
+        # issuing every launch from Python
+        self.enable_hybrid_graphs = (
+            str(dev) != "cpu" and getattr(self.model, "prenorm", False)
+            and bool(int(__import__("os").environ.get(
+                "POLYRL_HIP_GRAPHS", "1"))))
+        self._graph_seen: Dict[int, int] = {}
 
     # ------------------------------------------------------------ public API
     def add_request(self, rid: str, input_ids: List[int],
@@ -524,6 +532,9 @@ class Engine:
             self._kv_shape = (self.kv.num_pages, self.kv.page_size)
             self.kv.rows = {}
             self.states.tensors = {}
+            # captured steps hold pointers into the freed pools
+            self._graphs, self._graph_pool = {}, None
+            self._graph_seen = {}
             self._kv_released = True
             if str(self.device).startswith("cuda"):
                 torch.cuda.empty_cache()
@@ -795,6 +806,7 @@ class Engine:
         dev = self.device
         tok, pos, sot, cu, slots, sids, maps = [], [], [], [0], [], [], []
         prev = []
+        singles = all(len(it[2]) == 1 for it in items)   # a pure decode step
         for b, (r, start, toks) in enumerate(items):
             sid = self._seq_ids[r.rid]
             n = len(toks)
@@ -815,16 +827,26 @@ class Engine:
             cu.append(cu[-1] + n)
             slots.append(self.states.slot(sid))
             sids.append(sid)
-            maps.append(self.kv.slots_for(sid, start, n))
+            if singles:                 # plain integers, no tensor per row
+                ps = self.kv.page_size
+                maps.append(self.kv._seq_pages[sid][start // ps] * ps
+                            + start % ps)
+            else:
+                maps.append(self.kv.slots_for(sid, start, n))
         i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
         th = np.asarray(tok, dtype=np.int64)
+        pages = [self.kv._seq_pages[s] for s in sids]
+        ptab = np.zeros((len(sids), max(max(map(len, pages), default=1), 1)),
+                        dtype=np.int32)
+        for i, p in enumerate(pages):
+            ptab[i, :len(p)] = p
         return HybridBatch(
             tokens=torch.from_numpy(th).to(dev), tokens_host=th,
             prev_tokens=torch.tensor(prev, dtype=torch.int64, device=dev),
             positions=i32(pos), seq_of_tok=i32(sot), cu_q=i32(cu),
             state_slot=i32(slots),
-            slot_mapping=torch.cat(maps).to(dev),
-            page_table=self.kv.page_table(sids).to(dev),
+            slot_mapping=i32(maps) if singles else torch.cat(maps).to(dev),
+            page_table=torch.from_numpy(ptab).to(dev),
             attn_tiles=ops.seq.attention_tiles(
                 [len(it[2]) for it in items], dev)), cu
 
@@ -845,7 +867,10 @@ class Engine:
             not prefill_reqs and _tuned_decode_enabled()
             and ops.extension_loaded())
         try:
-            res = self.model.forward_batch(bt, self.kv, self.states)
+            if not prefill_reqs and self._graph_wanted(len(items)):
+                res = self._mixed_decode_graphed(bt, len(items))
+            else:
+                res = self.model.forward_batch(bt, self.kv, self.states)
         finally:
             hybrid_model.set_tuned_products(False)
         rows, reqs = [], []
@@ -860,6 +885,74 @@ class Engine:
         if reqs:
             idx = torch.tensor(rows, dtype=torch.long, device=self.device)
             self._sample_last(reqs, res.index_select(0, idx))
+
+    _GRAPH_AFTER = 2          # eager steps of a batch size before capture
+    _GRAPH_MAX = 12           # captured batch sizes kept
+
+    def _graph_wanted(self, B: int) -> bool:
+        """Capture a batch size once it has recurred (a size seen only in
+        passing, while requests finish one by one, stays eager)."""
+        if not self.enable_hybrid_graphs:
+            return False
+        if B in self._graphs:
+            return True
+        n = self._graph_seen.get(B, 0) + 1
+        self._graph_seen[B] = n
+        return n > self._GRAPH_AFTER and len(self._graphs) < self._GRAPH_MAX
+
+    def _mixed_decode_graphed(self, bt, B: int) -> torch.Tensor:
+        """A pure decode step (one token per sequence) as one hipGraph
+        replay.  The batch descriptors live in static device buffers that
+        every step overwrites; cache rows, state slots and weights are the
+        engine's own tensors, so the graph reads and writes them in place.
+        The warm-up run before the capture advances the recurrent states,
+        so they are saved and put back around it."""
+        from .hybrid_model import HybridBatch
+        dev = self.device
+        st = self._graphs.get(B)
+        if st is None:
+            i32, i64 = torch.int32, torch.int64
+            z = lambda *s, dt=i32: torch.zeros(*s, dtype=dt, device=dev)
+            sb = HybridBatch(
+                tokens=z(B, dt=i64), tokens_host=None,
+                prev_tokens=z(B, dt=i64), positions=z(B),
+                seq_of_tok=torch.arange(B, dtype=i32, device=dev),
+                cu_q=torch.arange(B + 1, dtype=i32, device=dev),
+                state_slot=z(B), slot_mapping=z(B),
+                page_table=z(B, max(self.kv.num_pages, 1)),
+                attn_tiles=(z(B), z(B), 1))
+            st = {"bt": sb}
+            self._load_static(sb, bt)
+            saved = {k: t.clone() for k, t in self.states.tensors.items()}
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                self.model.forward_batch(sb, self.kv, self.states)
+            torch.cuda.current_stream().wait_stream(side)
+            for k, t in self.states.tensors.items():
+                t.copy_(saved[k])
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, pool=self._graph_pool):
+                st["res"] = self.model.forward_batch(sb, self.kv, self.states)
+            if self._graph_pool is None:
+                self._graph_pool = g.pool()
+            st["graph"] = g
+            self._graphs[B] = st
+        self._load_static(st["bt"], bt)
+        st["graph"].replay()
+        return st["res"]
+
+    @staticmethod
+    def _load_static(sb, bt) -> None:
+        """Copy a step's batch descriptors into a captured step's buffers.
+        Page-table columns past this step's width keep older entries; no
+        row of the step reaches them."""
+        sb.tokens.copy_(bt.tokens)
+        sb.prev_tokens.copy_(bt.prev_tokens)
+        sb.positions.copy_(bt.positions)
+        sb.state_slot.copy_(bt.state_slot)
+        sb.slot_mapping.copy_(bt.slot_mapping)
+        sb.page_table[:, :bt.page_table.shape[1]].copy_(bt.page_table)
 
     @torch.no_grad()
     def step_forced(self, entries, end=()):

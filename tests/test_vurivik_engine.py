@@ -533,3 +533,35 @@ def test_registry_preset_runs_and_resumes_memory():
     assert not e.kv.rows
     e.resume_memory()
     torch.testing.assert_close(run(e, "b", t), a)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
+def test_decode_graph_replays_match_eager_steps(dt):
+    """Pure decode steps replay a captured graph once their batch size has
+    recurred: 40 greedy tokens (eager sampling, copies and a host sync
+    between the replays) equal the run with every launch issued eagerly,
+    also after the batch shrinks to another size."""
+    W = O.make_weights(FULL, seed=47)
+    prompts = [toks(n, seed=80 + n) for n in (9, 3, 14)]
+    new = (40, 17, 40)
+    outs = {}
+    for graphs in (False, True):
+        e = engine(FULL, W, ("cuda", dt), slots=3)
+        assert e.enable_hybrid_graphs
+        e.enable_hybrid_graphs = graphs
+        for i, (p, n) in enumerate(zip(prompts, new)):
+            e.add_request(f"g-{i}", p, SamplingParams(temperature=0.0,
+                                                      max_new_tokens=n))
+        got = {}
+        while e.has_work():
+            for o in e.step():
+                got[o.rid] = o
+        outs[graphs] = [got[f"g-{i}"] for i in range(3)]
+        assert sorted(e._graphs) == ([2, 3] if graphs else [])
+        assert e.states.free_slots == e.states.num_slots
+    for a, b in zip(outs[False], outs[True]):
+        assert a.output_ids == b.output_ids
+        torch.testing.assert_close(torch.tensor(a.output_logprobs),
+                                   torch.tensor(b.output_logprobs),
+                                   rtol=1e-5, atol=1e-5)
