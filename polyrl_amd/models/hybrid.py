@@ -1,10 +1,10 @@
 """Configuration of hybrid decoders: a stack whose layers each pick one
-sequence mixer (recurrent, state-space, gated linear attention, windowed
-latent attention or grouped-query attention) and one feed-forward (dense,
-table-routed experts, router-chosen experts, or none).
+sequence mixer (recurrent, state-space, gated linear attention, a real-gated
+linear recurrence, latent attention or grouped-query attention) and one
+feed-forward (dense, table-routed experts, router-chosen experts, or none).
 
 The Bizusun design is the first family described this way, Kuforax the
-second, Vurivik the third.  Everything that
+second, Vurivik the third, Nasipel the fourth.  Everything that
 can differ between two models of a family is a field here and is read from
 the checkpoint's ``config.json``; constants that the design fixes (the decay
 constant of the delta rule, its key epsilon) are defaults of the mixer
@@ -44,6 +44,21 @@ class GLASpec:
 
 
 @dataclass
+class RGLRUSpec:
+    """Recurrent block with a real-gated linear recurrent unit: a GELU
+    branch and a convolved branch of ``width`` channels each; the convolved
+    branch drives a per-channel recurrence whose decay gate and input gate
+    are block-diagonal (``blocks`` equal blocks); decay
+    ``a = exp(-decay_mult * r * softplus(lam))``, input scaled by
+    ``sqrt(1 - a^2)``."""
+    width: int
+    blocks: int
+    conv: int = 4
+    decay_mult: float = 8.0
+    kind: str = "rglru"
+
+
+@dataclass
 class SSMSpec:
     """Mamba-2 style selective state space layer."""
     heads: int
@@ -65,7 +80,14 @@ class SSMSpec:
 
 @dataclass
 class LatentAttnSpec:
-    """Windowed multi-head attention over a shared low-rank latent."""
+    """Multi-head attention over a shared low-rank latent, windowed or
+    (``window = UNBOUNDED``) causal.  Optional parts, each a parameter: a
+    normed low-rank latent for the queries (``q_rank`` > 0: tensors 'dq',
+    'dq.norm', 'uq' instead of 'q'), a learned logit per head in the softmax
+    denominator (``sink``), the output gate per entry (``gate="element"``,
+    'g' has heads * vdim rows) or per head (``gate="head"``, 'g' has one row
+    per head), and a rotation given as a :class:`RopeSpec` (``rope``:
+    interleaved pairs, YaRN) instead of plain rotate-half."""
     heads: int
     dim: int              # unrotated query/key size per head
     rot_dim: int          # rotated query/key size per head (key part shared)
@@ -76,17 +98,24 @@ class LatentAttnSpec:
     rope_base: float = 10000.0
     rope_dims: Optional[int] = None       # rotated pairs cover the first dims
     kv_from: Optional[int] = None         # reuse that layer's latent cache
+    q_rank: int = 0
+    sink: bool = True
+    gate: str = "element"
+    rope: Optional["RopeSpec"] = None
     kind: str = "latent_attention"
 
     def __post_init__(self):
+        if self.rope is not None:
+            self.rope_base, self.rope_dims = self.rope.base, self.rope.dims
         if self.rope_dims is None:
             self.rope_dims = self.rot_dim
 
 
 @dataclass
 class RopeSpec:
-    """Rotate-half rotary positions on the first ``dims`` entries of every
-    head.  ``factor`` > 1 switches on YaRN: pairs that turn fewer than
+    """Rotary positions on the first ``dims`` entries of every head; pair i
+    is (i, i + dims/2) (rotate-half) or, ``interleaved``, (2i, 2i + 1).
+    ``factor`` > 1 switches on YaRN: pairs that turn fewer than
     ``slow`` times within ``original`` positions have their frequency divided
     by ``factor``, pairs that turn more than ``fast`` times keep it, a linear
     ramp joins the two, and cos/sin are scaled by ``amp_slope*ln(factor)+1``."""
@@ -97,6 +126,7 @@ class RopeSpec:
     fast: float = 32.0
     slow: float = 1.0
     amp_slope: float = 0.1
+    interleaved: bool = False
 
     def inv_freq_and_amp(self):
         """(per-pair frequencies as Python floats, cos/sin amplitude)."""
@@ -134,7 +164,16 @@ class WindowAttnSpec:
     projections (``qkv_bias``), one learned logit per head that joins the
     softmax denominator and contributes no value row (``sink``), and a query
     temperature ``1 + q_temp_coef * ln(floor((p + 1) / q_temp_every) + 1)``
-    at position p.  ``window = UNBOUNDED`` is plain causal attention."""
+    at position p.  ``window = UNBOUNDED`` is plain causal attention.
+    Further parts: every query and key head divided by its root mean square
+    after the rotation (``head_unit_norm``, no weight), scores capped as
+    ``softcap * tanh(score / softcap)``, a learned number per head added to
+    the capped score (``head_bias``, tensor 'pb'), weights
+    ``sigmoid(score)`` per visible key instead of a softmax over the keys
+    (``weights="sigmoid"``), and values that are rotated by their position
+    over all ``vdim`` entries before they are cached, the head's sum being
+    turned back by the query's position (``value_rope_base`` > 0; pairs
+    (m, m + vdim/2), frequencies base^(-2m/vdim), never scaled)."""
     heads: int
     kv_heads: int
     dim: int
@@ -152,6 +191,11 @@ class WindowAttnSpec:
     head_gate: bool = False
     bias_far: float = 0.0
     bias_rows: Optional[int] = None       # rows of the table; None = tensor
+    head_unit_norm: bool = False
+    softcap: float = 0.0
+    head_bias: bool = False
+    weights: str = "softmax"
+    value_rope_base: float = 0.0
     kind: str = "attention"
 
     def bucket_of_distance(self) -> List[int]:
@@ -183,6 +227,15 @@ class FFSpec:
     group_keep: int = 1
     shared_ff: int = 0
     weight_eps: float = 1e-20
+    # routed_moe: the router's scores are a softmax over the experts or each
+    # logit's own sigmoid; a group's score is the sum of its best
+    # ``group_top`` choice scores; the normalised weights are multiplied by
+    # ``route_scale``; experts are W_down gelu(W_up h) ("gelu") or
+    # W_down (silu(W_gate h) * W_up h) ("silu_gated")
+    router_act: str = "softmax"
+    group_top: int = 1
+    route_scale: float = 1.0
+    expert_act: str = "gelu"
     # dense: "silu" is silu(gate) * up; "clamped" is g * sigmoid(slope * g)
     # * (u + shift) with g = min(gate, limit), u = clamp(up, -limit, limit)
     act: str = "silu"
@@ -224,8 +277,15 @@ class HybridConfig:
     # x += norm(ff(norm(x))) with per-channel weights stored as offsets
     # from ``norm_offset``.  "prenorm": x += m * mixer(norm(x)),
     # x += m * ff(norm(x)), x += m * token-side input, with per-channel
-    # weights and m = ``residual_mult``.
+    # weights and m = ``residual_mult``.  "parallel": both sublayers read
+    # the same stream, x += mixer(norm1(x)) + ff(norm2(x)).
     layer_style: str = "canon"
+    # "rms": x / sqrt(mean(x^2) + eps) * w.  "layer": (x - mean) /
+    # sqrt(var + eps) * w (no bias); parallel layers only.
+    norm_kind: str = "rms"
+    # every sublayer's result is multiplied by sigmoid(W h + b) of the
+    # sublayer's own input h (tensors 'rg1', 'rg1.b', 'rg2', 'rg2.b')
+    gated_residual: bool = False
     norm_offset: float = 0.0
     residual_mult: float = 1.0
     # the embedding: table row * embed_scale [+ hashed pair row]
@@ -294,6 +354,12 @@ class HybridConfig:
                                      "equal latent and rotated sizes")
             if m.kind == "gla":
                 assert m.heads > 0 and m.dim > 0 and m.vdim > 0 and m.tau > 0
+            if m.kind == "rglru":
+                assert m.width % m.blocks == 0 and m.conv >= 1
+            if m.kind == "latent_attention":
+                assert m.gate in ("element", "head")
+                if m.rope is not None:
+                    assert m.rope.dims % 2 == 0 and m.rope.dims <= m.rot_dim
             if m.kind == "mamba2":
                 assert m.heads % m.groups == 0
                 assert m.inner % m.norm_groups == 0
@@ -301,6 +367,15 @@ class HybridConfig:
                 assert m.heads % m.kv_heads == 0 and m.window >= 1
                 if m.rope is not None:
                     assert m.rope.dims % 2 == 0 and m.rope.dims <= m.dim
+                    if m.rope.interleaved:
+                        raise ValueError(f"layer {li}: grouped-query "
+                                         "attention rotates halves")
+                assert m.weights in ("softmax", "sigmoid")
+                if m.weights == "sigmoid" and (m.sink or m.bias_far > 0):
+                    raise ValueError(f"layer {li}: a sink or a distance "
+                                     "bias needs softmax weights")
+                if m.value_rope_base > 0:
+                    assert m.vdim % 2 == 0 and not m.values_from_keys
                 if m.bias_far > 0 and m.keep_first > 0:
                     raise ValueError(f"layer {li}: the distance bias covers "
                                      "the window only (no kept first tokens)")
@@ -315,6 +390,11 @@ class HybridConfig:
                 assert total % f.group_count == 0
                 assert 0 < f.group_keep <= f.group_count
                 assert 0 < f.top <= f.group_keep * (total // f.group_count)
+                assert f.router_act in ("softmax", "sigmoid")
+                assert f.expert_act in ("gelu", "silu_gated")
+                assert f.group_top >= 1
+        assert self.norm_kind == "rms" or self.layer_style == "parallel"
+        assert not self.gated_residual or self.layer_style == "parallel"
         if (self.loop_reinject or self.loop_step) and not self.loop:
             raise ValueError("pass inputs need a looped span")
         if self.loop is not None:
@@ -705,6 +785,154 @@ def vurivik_preset(width: int, layers: int, vocab: int = 32000,
         loop_step=bool(loop)).validate()
 
 
+def _rope_from_json(rot: Optional[dict], interleaved: bool = False
+                    ) -> Optional[RopeSpec]:
+    if not rot or int(rot.get("dims", 0)) <= 0:
+        return None
+    sc = rot.get("scaling") or {}
+    return RopeSpec(dims=int(rot["dims"]), base=float(rot["base"]),
+                    factor=float(sc.get("factor", 1.0)),
+                    original=float(sc.get("original", 0.0)),
+                    fast=float(sc.get("fast", 32.0)),
+                    slow=float(sc.get("slow", 1.0)),
+                    interleaved=interleaved)
+
+
+def _nasipel_mixer_from_json(kind: str, m: dict):
+    """Nasipel mixers: 'attention' (grouped-query, rotate-half rotation,
+    unit q/k heads, capped scores, sigmoid weights with a per-head bias,
+    rotated values), 'rglru' (gated linear recurrence) and
+    'latent_attention' (causal, query latent, interleaved YaRN rotation,
+    per-head output gate, no sink)."""
+    if kind == "rglru":
+        return RGLRUSpec(width=int(m["width"]), blocks=int(m["blocks"]),
+                         conv=int(m["conv"]))
+    if kind == "attention":
+        rot = m.get("rot") or {}
+        return WindowAttnSpec(
+            heads=int(m["heads"]), kv_heads=int(m["kv_heads"]),
+            dim=int(m["dim"]), vdim=int(m["vdim"]), window=UNBOUNDED,
+            scale=float(m["scale"]), rope=_rope_from_json(rot),
+            head_unit_norm=True, softcap=float(m.get("softcap") or 0.0),
+            head_bias=True, weights="sigmoid",
+            value_rope_base=float(rot.get("base", 10000.0)))
+    if kind == "latent_attention":
+        rope = _rope_from_json(m.get("rot"), interleaved=True)
+        return LatentAttnSpec(
+            heads=int(m["heads"]), dim=int(m["dim"]),
+            rot_dim=int(m["rot_dim"]), vdim=int(m["vdim"]),
+            kv_rank=int(m["kv_rank"]), window=UNBOUNDED,
+            scale=float(m["scale"]), q_rank=int(m["q_rank"]), sink=False,
+            gate="head", rope=rope)
+    raise ValueError(f"unknown mixer type {kind!r}")
+
+
+def _sigmoid_routed_ff_from_json(f: Optional[dict]) -> Optional[FFSpec]:
+    if f is None:
+        return None
+    if f["kind"] != "moe":
+        raise ValueError(f"unknown feed-forward kind {f['kind']!r}")
+    r = f["router"]
+    g = r.get("groups") or {}
+    return FFSpec(kind="routed_moe", ff=int(f["expert"]["ff"]),
+                  experts=int(r["experts"]), top=int(r["top"]),
+                  group_count=int(g.get("count", 1)),
+                  group_keep=int(g.get("keep", 1)),
+                  router_act="sigmoid", group_top=2,
+                  route_scale=float(r.get("scale", 1.0)),
+                  expert_act="silu_gated")
+
+
+def nasipel_config_from_json(d: dict) -> HybridConfig:
+    """Read a Nasipel ``config.json`` (already parsed)."""
+    layers = [HybridLayerSpec(_nasipel_mixer_from_json(L["type"], L["mixer"]),
+                              _sigmoid_routed_ff_from_json(L.get("mlp")))
+              for L in d["layers"]]
+    return HybridConfig(
+        arch="nasipel", vocab_size=int(d["vocab"]),
+        hidden_size=int(d["width"]), layers=layers,
+        norm_eps=float(d["norm"]["eps"]), canon_taps=1, token_side_dim=0,
+        layer_style="parallel", norm_kind="layer",
+        gated_residual=True).validate()
+
+
+def nasipel_config_to_json(cfg: HybridConfig) -> dict:
+    """Inverse of :func:`nasipel_config_from_json` (checkpoint export)."""
+    def rot_json(r):
+        out = {"base": r.base, "dims": r.dims}
+        if r.factor != 1.0:
+            out["scaling"] = {"factor": r.factor, "original": r.original,
+                              "fast": r.fast, "slow": r.slow}
+        return out
+    layers = []
+    for L in cfg.layers:
+        m = L.mixer
+        if m.kind == "rglru":
+            mj = {"width": m.width, "blocks": m.blocks, "conv": m.conv}
+        elif m.kind == "attention":
+            mj = {"heads": m.heads, "kv_heads": m.kv_heads, "dim": m.dim,
+                  "vdim": m.vdim, "scale": m.scale, "softcap": m.softcap,
+                  "rot": rot_json(m.rope) if m.rope is not None else
+                  {"base": m.value_rope_base, "dims": 0}}
+        else:
+            mj = {"heads": m.heads, "dim": m.dim, "rot_dim": m.rot_dim,
+                  "vdim": m.vdim, "kv_rank": m.kv_rank, "q_rank": m.q_rank,
+                  "scale": m.scale, "rot": rot_json(m.rope)}
+        fj = None
+        if L.ff is not None:
+            f = L.ff
+            fj = {"kind": "moe", "expert": {"ff": f.ff},
+                  "router": {"experts": f.experts, "top": f.top,
+                             "scale": f.route_scale,
+                             "groups": {"count": f.group_count,
+                                        "keep": f.group_keep}}}
+        layers.append({"type": m.kind, "mixer": mj, "mlp": fj})
+    return {"architecture": "Nasipel", "vocab": cfg.vocab_size,
+            "width": cfg.hidden_size, "layers": layers,
+            "norm": {"eps": cfg.norm_eps}}
+
+
+def nasipel_preset(width: int, layers: int, vocab: int = 32000,
+                   heads: int = 16, kv_heads: int = 4, experts: int = 16,
+                   top: int = 2, expert_ff: int = 0,
+                   pattern=("rglru", "rglru", "latent_attention",
+                            "attention")) -> HybridConfig:
+    """A Nasipel stack of realistic layer sizes (random weights): the mixer
+    kinds cycle through ``pattern``; every layer has sigmoid-routed gated
+    experts in two groups of which one stays open."""
+    hd = width // heads
+    expert_ff = expert_ff or max(64, width // 64 * 64)
+    groups = 2 if experts % 2 == 0 and experts // 2 >= top else 1
+    out = []
+    for li in range(layers):
+        kind = pattern[li % len(pattern)]
+        if kind == "rglru":
+            mixer = RGLRUSpec(width=width, blocks=heads, conv=4)
+        elif kind == "attention":
+            mixer = WindowAttnSpec(
+                heads=heads, kv_heads=kv_heads, dim=hd, vdim=hd,
+                window=UNBOUNDED, scale=1.0 / math.sqrt(hd),
+                rope=RopeSpec(dims=hd, base=10000.0), head_unit_norm=True,
+                softcap=30.0, head_bias=True, weights="sigmoid",
+                value_rope_base=10000.0)
+        else:
+            mixer = LatentAttnSpec(
+                heads=heads, dim=hd, rot_dim=hd // 2, vdim=hd,
+                kv_rank=4 * hd, window=UNBOUNDED,
+                scale=1.0 / math.sqrt(hd + hd // 2), q_rank=6 * hd,
+                sink=False, gate="head",
+                rope=RopeSpec(dims=hd // 2, base=10000.0, factor=4.0,
+                              original=4096.0, interleaved=True))
+        ff = FFSpec("routed_moe", expert_ff, experts, top,
+                    group_count=groups, group_keep=1, router_act="sigmoid",
+                    group_top=2, route_scale=1.5, expert_act="silu_gated")
+        out.append(HybridLayerSpec(mixer, ff))
+    return HybridConfig(arch="nasipel", vocab_size=vocab, hidden_size=width,
+                        layers=out, norm_eps=1e-5, canon_taps=1,
+                        token_side_dim=0, layer_style="parallel",
+                        norm_kind="layer", gated_residual=True).validate()
+
+
 def read_config_dir(path: str):
     """Model config from a checkpoint folder's ``config.json``.  The
     ``architecture`` key names the family; HF-style folders
@@ -718,6 +946,8 @@ def read_config_dir(path: str):
         return kuforax_config_from_json(d)
     if arch == "Vurivik":
         return vurivik_config_from_json(d)
+    if arch == "Nasipel":
+        return nasipel_config_from_json(d)
     mt = d.get("model_type")
     if mt in ("llama", "qwen2"):
         from .registry import DecoderConfig

@@ -107,8 +107,23 @@ MODEL_CONFIGS = {
 
 
 def _hybrid_presets():
-    from .hybrid import bizusun_preset, kuforax_preset, vurivik_preset
+    from .hybrid import (bizusun_preset, kuforax_preset, nasipel_preset,
+                         vurivik_preset)
     return {
+        # tiny stack for CPU unit tests / fast GPU smoke
+        "nasipel-debug": lambda: nasipel_preset(
+            width=64, layers=4, vocab=300, heads=4, kv_heads=2, experts=6,
+            top=2, expert_ff=32),
+        # bench pairs: beside llama-400m / llama3-1b / llama3-8b-l8
+        "nasipel-400m": lambda: nasipel_preset(
+            width=1024, layers=12, vocab=32000, heads=16, kv_heads=4,
+            experts=8, top=2, expert_ff=2048),
+        "nasipel-1b": lambda: nasipel_preset(
+            width=2048, layers=16, vocab=128256, heads=32, kv_heads=8,
+            experts=16, top=2, expert_ff=2560),
+        "nasipel-8b-l8": lambda: nasipel_preset(
+            width=4096, layers=8, vocab=128256, heads=32, kv_heads=8,
+            experts=16, top=2, expert_ff=3584),
         # tiny looped stack for CPU unit tests / fast GPU smoke
         "vurivik-debug": lambda: vurivik_preset(
             width=64, layers=4, vocab=300, heads=4, kv_heads=2, ff_mult=2.5,

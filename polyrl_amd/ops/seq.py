@@ -249,28 +249,34 @@ def rope_inv_freq(dims: int, base: float, device) -> torch.Tensor:
     return (base ** (-2.0 * i / dims)).float().to(device)
 
 
-def rope_partial_(q, offset: int, inv_freq, positions):
-    """Rotate-half RoPE in place on q[..., offset:offset+dims] of a
-    (N, H, Dh) tensor; angle = fp32(position) * inv_freq, fp32 cos/sin."""
+def rope_partial_(q, offset: int, inv_freq, positions, amp: float = 1.0,
+                  interleaved: bool = False):
+    """RoPE in place on q[..., offset:offset+dims] of a (N, H, Dh) tensor;
+    angle = fp32(position) * inv_freq, fp32 cos/sin times ``amp``; pairs are
+    (i, i + dims/2) or, ``interleaved``, (2i, 2i + 1)."""
     if q.is_cuda:
         if q.shape[0] and inv_freq.numel():
-            _ext().seq_rope_partial(q, offset, inv_freq, positions)
+            _ext().seq_rope_partial(q, offset, inv_freq, positions, amp,
+                                    interleaved)
         return q
-    return R.rope_partial_(q, offset, inv_freq, positions)
+    return R.rope_partial_(q, offset, inv_freq, positions, amp, interleaved)
 
 
 def latent_kv_store(dkv, rank: int, norm_w, eps: float, positions, inv_freq,
-                    cache, slot_mapping) -> None:
+                    cache, slot_mapping, amp: float = 1.0,
+                    interleaved: bool = False) -> None:
     """Row n of dkv = [latent (rank) | shared key part]: RMS-norm the latent
-    (times norm_w), rotate the key part, and write both into the paged
-    latent cache (pages, page_size, rank+rot) at slot_mapping[n]."""
+    (times norm_w), rotate the key part (pairs and amplitude as in
+    :func:`rope_partial_`), and write both into the paged latent cache
+    (pages, page_size, rank+rot) at slot_mapping[n]."""
     if dkv.is_cuda:
         if dkv.shape[0]:
             _ext().seq_latent_kv_store(dkv, rank, norm_w, eps, positions,
-                                       inv_freq, cache, slot_mapping)
+                                       inv_freq, cache, slot_mapping, amp,
+                                       interleaved)
         return
     R.latent_kv_store(dkv, rank, norm_w, eps, positions, inv_freq, cache,
-                      slot_mapping)
+                      slot_mapping, amp, interleaved)
 
 
 def attention_tiles(lens, device):
@@ -294,9 +300,12 @@ def latent_window_attention(q_lat, q_rot, cache, page_table, seq_of_tok,
                             out_dtype, tiles=None) -> torch.Tensor:
     """Windowed attention of every row against its sequence's paged latent
     cache: score_j = (q_lat . c_j + q_rot . kr_j) * scale for
-    0 <= pos - j < window; softmax whose denominator also holds exp(sink_h);
-    returns sum_j p_j c_j, (N, H, rank).  All heads share the cache rows."""
+    0 <= pos - j < window; softmax whose denominator also holds exp(sink_h)
+    when ``sink`` (H,) is given; returns sum_j p_j c_j, (N, H, rank).  All
+    heads share the cache rows."""
     row = q_lat.shape[2] + q_rot.shape[2]
+    if q_lat.is_cuda and sink is None:
+        sink = torch.Tensor()
     if q_lat.is_cuda and tiles is not None and q_lat.shape[0] and \
             q_lat.dtype == torch.bfloat16 and row % 8 == 0 and row <= 576:
         out = torch.empty(q_lat.shape, dtype=out_dtype, device=q_lat.device)
@@ -319,7 +328,8 @@ def latent_window_attention(q_lat, q_rot, cache, page_table, seq_of_tok,
 
 def gqa_prepare_store(q, k, v, q_norm, k_norm, eps: float, inv_freq,
                       amp: float, positions, cache, slot_mapping, H: int,
-                      G: int, D: int, Dv: int) -> torch.Tensor:
+                      G: int, D: int, Dv: int, head_unit: bool = False,
+                      v_inv_freq=None) -> torch.Tensor:
     """Queries and cache rows of grouped-query attention from a step's
     projections (column slices allowed).  Optional RMS norm over the WHOLE
     query row and the whole key row (weights q_norm / k_norm), then
@@ -327,7 +337,11 @@ def gqa_prepare_store(q, k, v, q_norm, k_norm, eps: float, inv_freq,
     angle fp32(position)*inv_freq and cos/sin scaled by ``amp``.  The cache
     row of a token, (pages, page_size, G*D + G*Dv) at slot_mapping[n], is
     [keys (normed, rotated) | values]; values are ``v`` or, when ``v`` is
-    None, the key projection as it came in.  Returns the queries (N, H*D)."""
+    None, the key projection as it came in.  ``head_unit`` divides every
+    query and key head by its root mean square after the rotation (no
+    weight); ``v_inv_freq`` (Dv/2,) rotates every value head over all its
+    entries by its position (pairs (m, m + Dv/2)) before it is cached.
+    Returns the queries (N, H*D)."""
     if q.is_cuda:
         out = torch.empty(q.shape[0], H * D, dtype=q.dtype, device=q.device)
         if q.shape[0]:
@@ -337,10 +351,12 @@ def gqa_prepare_store(q, k, v, q_norm, k_norm, eps: float, inv_freq,
                 q_norm if q_norm is not None else e,
                 k_norm if k_norm is not None else e, eps,
                 inv_freq if inv_freq is not None else e, amp, positions,
-                cache, slot_mapping, H, G, D, Dv)
+                cache, slot_mapping, H, G, D, Dv, head_unit,
+                v_inv_freq if v_inv_freq is not None else e)
         return out
     return R.gqa_prepare_store(q, k, v, q_norm, k_norm, eps, inv_freq, amp,
-                               positions, cache, slot_mapping, H, G, D, Dv)
+                               positions, cache, slot_mapping, H, G, D, Dv,
+                               head_unit, v_inv_freq)
 
 
 def gqa_window_attention(q, cache, page_table, seq_of_tok, positions, H: int,
@@ -348,15 +364,23 @@ def gqa_window_attention(q, cache, page_table, seq_of_tok, positions, H: int,
                          keep_first: int, rel, dist_bucket, gate,
                          scale: float, out_dtype, tiles=None, sink=None,
                          q_temp_coef: float = 0.0,
-                         q_temp_every: int = 1) -> torch.Tensor:
-    """Softmax attention of every row against its sequence's paged K/V rows
+                         q_temp_every: int = 1, softcap: float = 0.0,
+                         head_bias=None, sigmoid_weights: bool = False,
+                         v_inv_freq=None) -> torch.Tensor:
+    """Attention of every row against its sequence's paged K/V rows
     (layout of :func:`gqa_prepare_store`).  Row at position p sees key j if
     j <= p and (p - j < window or j < keep_first).  score = q.k * scale
     * (1 + q_temp_coef * ln(floor((p + 1) / q_temp_every) + 1))
     [+ rel[dist_bucket[p - j], head]]; with ``sink`` (H,) fp32 the
     denominator also holds exp(sink[h]) once; ``gate`` (N, H) multiplies
     head h's output by sigmoid(gate[n, h]).  Query head h reads key/value
-    head h // (H // G).  Returns (N, H*Dv)."""
+    head h // (H // G).  ``softcap`` > 0 replaces the score by
+    softcap * tanh(score / softcap); ``head_bias`` (H,) fp32 is added after
+    that; with ``sigmoid_weights`` a visible key weighs
+    sigmoid(score) instead of its softmax share (no normalisation over
+    keys); ``v_inv_freq`` (Dv/2,) turns every head's sum back by the row's
+    position (the inverse of the value rotation of
+    :func:`gqa_prepare_store`) before the gate.  Returns (N, H*Dv)."""
     if q.is_cuda:
         out = torch.empty(q.shape[0], H * Dv, dtype=out_dtype,
                           device=q.device)
@@ -367,7 +391,10 @@ def gqa_window_attention(q, cache, page_table, seq_of_tok, positions, H: int,
                     dist_bucket if dist_bucket is not None else e,
                     gate if gate is not None else e, scale,
                     sink if sink is not None else e, q_temp_coef,
-                    q_temp_every)
+                    q_temp_every, softcap,
+                    head_bias if head_bias is not None else e,
+                    sigmoid_weights,
+                    v_inv_freq if v_inv_freq is not None else e)
             if tiles is not None and tiles[2] == 0 and \
                     gqa_mfma_supported(q, D, Dv):
                 _ext().seq_gqa_window_attention_mfma(out, q, tiles[0],
@@ -378,7 +405,8 @@ def gqa_window_attention(q, cache, page_table, seq_of_tok, positions, H: int,
     return R.gqa_window_attention(q, cache, page_table, seq_of_tok, positions,
                                   H, G, D, Dv, window, keep_first, rel,
                                   dist_bucket, gate, scale, out_dtype, sink,
-                                  q_temp_coef, q_temp_every)
+                                  q_temp_coef, q_temp_every, softcap,
+                                  head_bias, sigmoid_weights, v_inv_freq)
 
 
 def gqa_mfma_supported(q, D: int, Dv: int) -> bool:
@@ -389,20 +417,24 @@ def gqa_mfma_supported(q, D: int, Dv: int) -> bool:
             and D <= 128 and Dv <= 128)
 
 
-def moe_route(logits, correction, top: int, groups: int, keep: int):
-    """Router choice for every row of fp32 logits (N, E): s = softmax,
+def moe_route(logits, correction, top: int, groups: int, keep: int,
+              act: str = "softmax", group_top: int = 1):
+    """Router choice for every row of fp32 logits (N, E): s = softmax (or,
+    ``act="sigmoid"``, the logistic function of every logit on its own),
     choice score = s + correction; experts form ``groups`` equal groups of
-    neighbours, only the ``keep`` groups with the largest best choice score
-    stay eligible; the ``top`` largest eligible choice scores win.  Returns
+    neighbours, a group's score is the sum of its ``group_top`` largest
+    choice scores, only the ``keep`` groups with the largest score stay
+    eligible; the ``top`` largest eligible choice scores win.  Returns
     (index int32 (N, top), s at those indices fp32 (N, top))."""
     if logits.is_cuda:
         N = logits.shape[0]
         idx = torch.empty(N, top, dtype=torch.int32, device=logits.device)
         w = torch.empty(N, top, dtype=torch.float32, device=logits.device)
         if N:
-            _ext().seq_moe_route(idx, w, logits, correction, groups, keep)
+            _ext().seq_moe_route(idx, w, logits, correction, groups, keep,
+                                 {"softmax": 0, "sigmoid": 1}[act], group_top)
         return idx, w
-    return R.moe_route(logits, correction, top, groups, keep)
+    return R.moe_route(logits, correction, top, groups, keep, act, group_top)
 
 
 def gelu_erf(x):
@@ -420,35 +452,37 @@ def moe_routed_ffn_supported(h, top: int, ff: int) -> bool:
     return moe_table_ffn_supported(h, top, ff)
 
 
-def moe_routed_ffn(h, idx, w_up, w_down) -> torch.Tensor:
-    """Router-chosen plain experts: row t*top+k of the result is expert
-    idx[t, k] applied to h[t], W_down gelu_erf(W_up h); rows whose index is
-    >= E (identity experts) are left unwritten.  w_up (E, ff, W), w_down
-    (E, W, ff)."""
+def moe_routed_ffn(h, idx, w_up, w_down, gated: bool = False) -> torch.Tensor:
+    """Router-chosen experts: row t*top+k of the result is expert
+    idx[t, k] applied to h[t]; rows whose index is >= E (identity experts)
+    are left unwritten.  Plain experts: W_down gelu_erf(W_up h) with w_up
+    (E, ff, W); ``gated``: W_down (silu(W_gate h) * W_up h) with w_up
+    (E, 2*ff, W) holding gate rows then up rows.  w_down (E, W, ff)."""
     if h.is_cuda:
         N, top = idx.shape
         y = torch.empty(N * top, h.shape[1], dtype=h.dtype, device=h.device)
         act = torch.empty(N * top, w_down.shape[2], dtype=h.dtype,
                           device=h.device)
-        _ext().seq_moe_routed_ffn(y, act, h, idx, w_up, w_down)
+        _ext().seq_moe_routed_ffn(y, act, h, idx, w_up, w_down, gated)
         return y
-    return R.moe_routed_ffn(h, idx, w_up, w_down)
+    return R.moe_routed_ffn(h, idx, w_up, w_down, gated)
 
 
 def moe_weighted_combine(ys, idx, w, h, shared, E: int, weight_eps: float,
-                         out_dtype) -> torch.Tensor:
+                         out_dtype, scale: float = 1.0) -> torch.Tensor:
     """y[n] = sum_k w'[n,k] * (ys[n*top+k] if idx[n,k] < E else h[n])
-    [+ shared[n]] with w' = w / (sum_k w + weight_eps), fp32 sums."""
+    [+ shared[n]] with w' = scale * w / (sum_k w + weight_eps), fp32
+    sums."""
     if ys.is_cuda:
         out = torch.empty(h.shape, dtype=out_dtype, device=h.device)
         if h.shape[0]:
             _ext().seq_moe_weighted_combine(
                 out, ys, idx, w, h,
                 shared if shared is not None else torch.Tensor(), E,
-                weight_eps)
+                weight_eps, scale)
         return out
     return R.moe_weighted_combine(ys, idx, w, h, shared, E, weight_eps,
-                                  out_dtype)
+                                  out_dtype, scale)
 
 
 def silu_mul_any(gate, up):
@@ -480,6 +514,58 @@ def sigmoid_mul(x, gate):
             _ext().seq_act_mul(out, gate, x, 1, 0.0, 0.0, 0.0)
         return out
     return R.sigmoid_mul(x, gate)
+
+
+def sigmoid_mul_heads(x, gate):
+    """x (N, H*Dv) with head h's entries times sigmoid(gate[n, h])."""
+    if x.is_cuda:
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+        if x.shape[0]:
+            _ext().seq_sigmoid_mul_heads(out, x, gate)
+        return out
+    return R.sigmoid_mul_heads(x, gate)
+
+
+def gated_add_layernorm(res, y1, g1, y2, g2, w1, w2, eps: float, out_dtype):
+    """The joint of a layer whose two sublayers read the same stream:
+    res (N, D) fp32 += y1 * sigmoid(g1) [+ y2 * sigmoid(g2)] in place (a
+    missing gate means a plain add, a missing y1 no add), then the layer
+    norm of the new row, (x - mean) / sqrt(var + eps), once with each of
+    the weights w1 and w2 (D,) fp32: the two norms share their statistics.
+    Returns (h1, h2) in out_dtype; h2 is None without w2, both without
+    w1."""
+    if res.is_cuda:
+        e = torch.Tensor()
+        new = lambda: torch.empty(res.shape, dtype=out_dtype,
+                                  device=res.device)
+        h1 = new() if w1 is not None else None
+        h2 = new() if w2 is not None else None
+        if res.shape[0]:
+            o = lambda t: t if t is not None else e
+            _ext().seq_gated_add_layernorm(o(h1), o(h2), res, o(y1), o(g1),
+                                           o(y2), o(g2), o(w1), o(w2), eps)
+        return h1, h2
+    return R.gated_add_layernorm(res, y1, g1, y2, g2, w1, w2, eps, out_dtype)
+
+
+def rglru_scan(u, gates, gate_bias, lam, y_lin, state, cu_q, state_slot,
+               decay_mult: float, out_dtype) -> torch.Tensor:
+    """Real-gated linear recurrence over packed rows; ``state`` (slots, C)
+    fp32 in place.  Channels form B equal blocks of bw; ``gates`` (B, N,
+    2*bw) fp32 holds the block-diagonal products for the decay gate (first
+    bw) and the input gate, ``gate_bias`` (B, 2*bw) their biases.  Per
+    channel: r = sigmoid(.), i = sigmoid(.), log a = -decay_mult * r *
+    softplus(lam), S <- a S + sqrt(1 - a^2) * i * u; returns
+    S * gelu_tanh(y_lin) (N, C).  ``u`` and ``y_lin`` may be column
+    slices."""
+    if u.is_cuda:
+        out = torch.empty(u.shape, dtype=out_dtype, device=u.device)
+        if u.shape[0]:
+            _ext().seq_rglru_scan(out, u, gates, gate_bias, lam, y_lin, state,
+                                  cu_q, state_slot, decay_mult)
+        return out
+    return R.rglru_scan(u, gates, gate_bias, lam, y_lin, state, cu_q,
+                        state_slot, decay_mult, out_dtype)
 
 
 def tanh_act(x):

@@ -192,34 +192,44 @@ def clamped_glu(gate, up, limit, slope, shift):
     return (g * torch.sigmoid(slope * g) * (u + shift)).to(gate.dtype)
 
 
-def _rotate(x, positions, inv_freq):
-    """x (N, ..., dims) rotate-half over the last axis."""
+def _rotate(x, positions, inv_freq, amp=1.0, interleaved=False,
+            negate=False):
+    """x (N, ..., dims) rotated over the last axis by position * inv_freq;
+    pairs are (i, i + dims/2) or, interleaved, (2i, 2i + 1); cos and sin
+    times ``amp``; ``negate`` turns the other way."""
     half = inv_freq.numel()
     ang = positions.float().unsqueeze(-1) * inv_freq.float()   # (N, half)
     while ang.dim() < x.dim():
         ang = ang.unsqueeze(1)
-    c, s = torch.cos(ang), torch.sin(ang)
+    c, s = torch.cos(ang) * amp, torch.sin(ang) * amp
+    if negate:
+        s = -s
+    if interleaved:
+        a, b = x[..., 0:2 * half:2].float(), x[..., 1:2 * half:2].float()
+        return torch.stack([a * c - b * s, b * c + a * s], -1).flatten(-2)
     a, b = x[..., :half].float(), x[..., half:2 * half].float()
     return torch.cat([a * c - b * s, b * c + a * s], -1)
 
 
-def rope_partial_(q, offset, inv_freq, positions):
+def rope_partial_(q, offset, inv_freq, positions, amp=1.0, interleaved=False):
     dims = 2 * inv_freq.numel()
     if dims == 0:
         return q
     part = q[..., offset:offset + dims]
-    part.copy_(_rotate(part, positions, inv_freq).to(q.dtype))
+    part.copy_(_rotate(part, positions, inv_freq, amp, interleaved)
+               .to(q.dtype))
     return q
 
 
 def latent_kv_store(dkv, rank, norm_w, eps, positions, inv_freq, cache,
-                    slot_mapping):
+                    slot_mapping, amp=1.0, interleaved=False):
     c = dkv[:, :rank].float()
     c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * norm_w.float()
     kr = dkv[:, rank:].float().clone()
     dims = 2 * inv_freq.numel()
     if dims:
-        kr[:, :dims] = _rotate(kr[:, :dims], positions, inv_freq)
+        kr[:, :dims] = _rotate(kr[:, :dims], positions, inv_freq, amp,
+                               interleaved)
     flat = cache.view(-1, cache.shape[-1])
     flat[slot_mapping.long()] = torch.cat([c, kr], -1).to(cache.dtype)
 
@@ -238,8 +248,11 @@ def latent_window_attention(q_lat, q_rot, cache, page_table, seq_of_tok,
         kv = flat[rows]                                  # (L, R + rd)
         s = (q_lat[n].float() @ kv[:, :R].t()
              + q_rot[n].float() @ kv[:, R:].t()) * scale   # (H, L)
-        s = torch.cat([s, sink.float().view(H, 1)], 1)
-        pr = torch.softmax(s, -1)[:, :-1]
+        if sink is not None:
+            s = torch.cat([s, sink.float().view(H, 1)], 1)
+            pr = torch.softmax(s, -1)[:, :-1]
+        else:
+            pr = torch.softmax(s, -1)
         out[n] = pr @ kv[:, :R]
     return out.to(out_dtype)
 
@@ -288,7 +301,8 @@ def gelu_erf(x):
 
 
 def gqa_prepare_store(q, k, v, q_norm, k_norm, eps, inv_freq, amp, positions,
-                      cache, slot_mapping, H, G, D, Dv):
+                      cache, slot_mapping, H, G, D, Dv, head_unit=False,
+                      v_inv_freq=None):
     N = q.shape[0]
     qf, kf = q.float(), k.float()
     vf = kf if v is None else v.float()
@@ -307,6 +321,11 @@ def gqa_prepare_store(q, k, v, q_norm, k_norm, eps, inv_freq, amp, positions,
             a, b = t[..., :half].clone(), t[..., half:2 * half].clone()
             t[..., :half] = a * c - b * s
             t[..., half:2 * half] = b * c + a * s
+    if head_unit:
+        qf = qf * torch.rsqrt(qf.pow(2).mean(-1, keepdim=True) + eps)
+        kf = kf * torch.rsqrt(kf.pow(2).mean(-1, keepdim=True) + eps)
+    if v_inv_freq is not None and v_inv_freq.numel():
+        vf = _rotate(vf.reshape(N, G, Dv), positions, v_inv_freq)
     flat = cache.view(-1, cache.shape[-1])
     flat[slot_mapping.long()] = torch.cat(
         [kf.reshape(N, G * D), vf.reshape(N, G * Dv)], -1).to(cache.dtype)
@@ -316,7 +335,8 @@ def gqa_prepare_store(q, k, v, q_norm, k_norm, eps, inv_freq, amp, positions,
 def gqa_window_attention(q, cache, page_table, seq_of_tok, positions, H, G,
                          D, Dv, window, keep_first, rel, dist_bucket, gate,
                          scale, out_dtype, sink=None, q_temp_coef=0.0,
-                         q_temp_every=1):
+                         q_temp_every=1, softcap=0.0, head_bias=None,
+                         sigmoid_weights=False, v_inv_freq=None):
     N = q.shape[0]
     ps = cache.shape[1]
     flat = cache.view(-1, cache.shape[-1]).float()
@@ -340,24 +360,36 @@ def gqa_window_attention(q, cache, page_table, seq_of_tok, positions, H, G,
         if rel is not None:
             dist = torch.tensor([p - j for j in js], dtype=torch.long)
             s = s + rel.float()[dist_bucket.long()[dist]].t()
-        if sink is not None:
+        if softcap > 0:
+            s = softcap * torch.tanh(s / softcap)
+        if head_bias is not None:
+            s = s + head_bias.float().view(H, 1)
+        if sigmoid_weights:
+            pr = torch.sigmoid(s)
+        elif sink is not None:
             pr = torch.softmax(
                 torch.cat([s, sink.float().view(H, 1)], 1), -1)[:, :-1]
         else:
             pr = torch.softmax(s, -1)
         o = torch.einsum("hj,jhv->hv", pr, vv)
+        if v_inv_freq is not None and v_inv_freq.numel():
+            o = _rotate(o.unsqueeze(0), torch.tensor([p]), v_inv_freq,
+                        negate=True)[0]
         if gate is not None:
             o = o * torch.sigmoid(gate[n].float()).unsqueeze(-1)
         out[n] = o
     return out.view(N, H * Dv).to(out_dtype)
 
 
-def moe_route(logits, correction, top, groups, keep):
-    s = torch.softmax(logits.float(), -1)
+def moe_route(logits, correction, top, groups, keep, act="softmax",
+              group_top=1):
+    s = torch.softmax(logits.float(), -1) if act == "softmax" \
+        else torch.sigmoid(logits.float())
     choice = s + correction.float()
     N, E = s.shape
     if groups > 1:
-        best = choice.view(N, groups, E // groups).max(-1).values
+        per = choice.view(N, groups, E // groups)
+        best = per.topk(min(group_top, E // groups), -1).values.sum(-1)
         kept = best.topk(keep, -1).indices
         open_ = torch.zeros(N, groups, dtype=torch.bool, device=s.device)
         open_.scatter_(1, kept, True)
@@ -367,7 +399,7 @@ def moe_route(logits, correction, top, groups, keep):
     return idx.int(), s.gather(1, idx)
 
 
-def moe_routed_ffn(h, idx, w_up, w_down):
+def moe_routed_ffn(h, idx, w_up, w_down, gated=False):
     N, top = idx.shape
     E = w_up.shape[0]
     y = torch.zeros(N * top, h.shape[1], dtype=h.dtype, device=h.device)
@@ -376,14 +408,20 @@ def moe_routed_ffn(h, idx, w_up, w_down):
         if e >= E:
             continue
         sl = (flat == e).nonzero().squeeze(1)
-        a = gelu_erf(h[sl // top] @ w_up[e].t())
+        a = h[sl // top] @ w_up[e].t()
+        if gated:
+            ff = w_down.shape[2]
+            a = silu_mul_any(a[:, :ff], a[:, ff:])
+        else:
+            a = gelu_erf(a)
         y[sl] = a @ w_down[e].t()
     return y
 
 
-def moe_weighted_combine(ys, idx, w, h, shared, E, weight_eps, out_dtype):
+def moe_weighted_combine(ys, idx, w, h, shared, E, weight_eps, out_dtype,
+                         scale=1.0):
     N, top = idx.shape
-    wn = w.float() / (w.float().sum(-1, keepdim=True) + weight_eps)
+    wn = w.float() / (w.float().sum(-1, keepdim=True) + weight_eps) * scale
     rows = ys.float().view(N, top, -1)
     ident = (idx >= E).unsqueeze(-1)
     rows = torch.where(ident, h.float().unsqueeze(1).expand_as(rows), rows)
@@ -391,3 +429,54 @@ def moe_weighted_combine(ys, idx, w, h, shared, E, weight_eps, out_dtype):
     if shared is not None:
         y = y + shared.float()
     return y.to(out_dtype)
+
+
+def sigmoid_mul_heads(x, gate):
+    N, H = gate.shape
+    return (x.float().view(N, H, -1)
+            * torch.sigmoid(gate.float()).unsqueeze(-1)
+            ).view(N, -1).to(x.dtype)
+
+
+def gated_add_layernorm(res, y1, g1, y2, g2, w1, w2, eps, out_dtype):
+    if y1 is not None:
+        add = y1.float() * torch.sigmoid(g1.float()) if g1 is not None \
+            else y1.float()
+        if y2 is not None:
+            add = add + (y2.float() * torch.sigmoid(g2.float())
+                         if g2 is not None else y2.float())
+        res.add_(add)
+    if w1 is None:
+        return None, None
+    d = res - res.mean(-1, keepdim=True)
+    unit = d * torch.rsqrt(d.pow(2).mean(-1, keepdim=True) + eps)
+    return ((unit * w1.float()).to(out_dtype),
+            None if w2 is None else (unit * w2.float()).to(out_dtype))
+
+
+def gelu_tanh(z):
+    c = math.sqrt(2.0 / math.pi)
+    return 0.5 * z * (1.0 + torch.tanh(c * (z + 0.044715 * z ** 3)))
+
+
+def rglru_scan(u, gates, gate_bias, lam, y_lin, state, cu_q, state_slot,
+               decay_mult, out_dtype):
+    N, C = u.shape
+    B, bw = gate_bias.shape[0], gate_bias.shape[1] // 2
+    g = gates.float() + gate_bias.float().unsqueeze(1)       # (B, N, 2bw)
+    r = torch.sigmoid(g[..., :bw]).permute(1, 0, 2).reshape(N, C)
+    i = torch.sigmoid(g[..., bw:]).permute(1, 0, 2).reshape(N, C)
+    log_a = -decay_mult * r * torch.nn.functional.softplus(
+        lam.float(), threshold=1e9)
+    a = torch.exp(log_a)
+    drive = torch.sqrt(1.0 - a * a) * i * u.float()
+    y = gelu_tanh(y_lin.float())
+    out = torch.empty(N, C, dtype=torch.float32, device=u.device)
+    cu = cu_q.tolist()
+    for b, slot in enumerate(state_slot.tolist()):
+        S = state[slot]
+        for n in range(cu[b], cu[b + 1]):
+            S = a[n] * S + drive[n]
+            out[n] = S * y[n]
+        state[slot] = S
+    return out.to(out_dtype)

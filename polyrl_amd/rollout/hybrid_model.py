@@ -160,6 +160,64 @@ class GLAMixer(_Part):
         return _mm(y, self.wo)
 
 
+class RGLRUMixer(_Part):
+    """Real-gated linear recurrence (models.hybrid.RGLRUSpec): one fused
+    projection (with biases) for the GELU branch and the convolved branch;
+    the stateful convolution; the block-diagonal gate products as one
+    batched fp32 product over the blocks (decay-gate rows then input-gate
+    rows of a block); one kernel for gates, decay, recurrence and the
+    product with the GELU branch.  State per sequence: the recurrence's
+    vector (fp32) and the convolution's last taps-1 inputs."""
+
+    def __init__(self, spec, width, device, dtype):
+        self.spec = s = spec
+        C, B = s.width, s.blocks
+        self.bw = bw = C // B
+        z = lambda *a, dt=dtype: torch.empty(*a, device=device, dtype=dt)
+        f32 = torch.float32
+        self.w_in = z(2 * C, width)
+        self.b_in = z(2 * C)
+        self.conv = z(C, s.conv, dt=f32)
+        self.conv_b = z(C, dt=f32)
+        self.w_gate = z(B, 2 * bw, bw, dt=f32)
+        self.b_gate = z(B, 2 * bw, dt=f32)
+        self.lam = z(C, dt=f32)
+        self.wo = z(width, C)
+
+    def named(self, p):
+        C, bw = self.spec.width, self.bw
+        return {p + "y": self.w_in[:C], p + "x": self.w_in[C:],
+                p + "y.b": self.b_in[:C], p + "x.b": self.b_in[C:],
+                p + "conv": self.conv, p + "conv.b": self.conv_b,
+                p + "ra": self.w_gate[:, :bw], p + "ri": self.w_gate[:, bw:],
+                p + "ra.b": self.b_gate[:, :bw],
+                p + "ri.b": self.b_gate[:, bw:],
+                p + "lam": self.lam, p + "o": self.wo}
+
+    def state_shapes(self):
+        s = self.spec
+        out = {"S": (s.width,)}
+        if s.conv > 1:
+            out["conv"] = (s.conv - 1, s.width)
+        return out
+
+    def forward(self, h, bt, li, model, cache, states):
+        s = self.spec
+        C, B, bw, N = s.width, s.blocks, self.bw, h.shape[0]
+        proj = _mm(h, self.w_in, self.b_in)
+        u = seq.causal_conv_state(proj.narrow(1, C, C), self.conv,
+                                  self.conv_b,
+                                  model._state(states, (li, "conv"), C),
+                                  bt.cu_q, bt.state_slot, bt.seq_of_tok,
+                                  False, False, h.dtype)
+        gates = torch.bmm(u.float().view(N, B, bw).transpose(0, 1),
+                          self.w_gate.transpose(1, 2))      # (B, N, 2bw)
+        y = seq.rglru_scan(u, gates, self.b_gate, self.lam,
+                           proj.narrow(1, 0, C), states.tensors[(li, "S")],
+                           bt.cu_q, bt.state_slot, s.decay_mult, h.dtype)
+        return _mm(y, self.wo)
+
+
 class SSMMixer(_Part):
     def __init__(self, spec, width, device, dtype):
         self.spec = spec
@@ -215,23 +273,42 @@ class LatentAttnMixer(_Part):
         self.nv = s.heads * s.vdim
         self.owner = s.kv_from is None
         self.row = s.kv_rank + s.rot_dim
-        # one projection for queries, output gate and (if owned) the latent
-        self.w_in = z(self.nq + self.nv + (self.row if self.owner else 0),
+        # rows of the fused input projection: the queries (or their latent),
+        # the output gate (per entry or per head) and (if owned) the latent
+        self.n0 = s.q_rank if s.q_rank > 0 else self.nq
+        self.ng = self.nv if s.gate == "element" else s.heads
+        self.w_in = z(self.n0 + self.ng + (self.row if self.owner else 0),
                       width)
+        self.dq_norm = z(s.q_rank, dt=f32) if s.q_rank > 0 else None
+        self.uq = z(self.nq, s.q_rank) if s.q_rank > 0 else None
         self.dkv_norm = z(s.kv_rank, dt=f32) if self.owner else None
         self.uk = z(s.heads * s.dim, s.kv_rank)
         self.uv = z(s.heads * s.vdim, s.kv_rank)
-        self.sink = z(s.heads, dt=f32)
+        self.sink = z(s.heads, dt=f32) if s.sink else None
         self.wo = z(width, self.nv)
-        self.inv_freq = seq.rope_inv_freq(s.rope_dims, s.rope_base, device)
+        self.amp, self.interleaved = 1.0, False
+        if s.rope is not None:
+            f, self.amp = s.rope.inv_freq_and_amp()
+            self.inv_freq = torch.tensor(f, dtype=torch.float64).float() \
+                .to(device)
+            self.interleaved = s.rope.interleaved
+        else:
+            self.inv_freq = seq.rope_inv_freq(s.rope_dims, s.rope_base,
+                                              device)
 
     def named(self, p):
-        out = {p + "q": self.w_in[:self.nq],
-               p + "g": self.w_in[self.nq:self.nq + self.nv],
-               p + "uk": self.uk, p + "uv": self.uv, p + "sink": self.sink,
-               p + "o": self.wo}
+        a, b = self.n0, self.n0 + self.ng
+        out = {p + "g": self.w_in[a:b],
+               p + "uk": self.uk, p + "uv": self.uv, p + "o": self.wo}
+        if self.uq is not None:
+            out.update({p + "dq": self.w_in[:a], p + "dq.norm": self.dq_norm,
+                        p + "uq": self.uq})
+        else:
+            out[p + "q"] = self.w_in[:a]
+        if self.sink is not None:
+            out[p + "sink"] = self.sink
         if self.owner:
-            out[p + "dkv"] = self.w_in[self.nq + self.nv:]
+            out[p + "dkv"] = self.w_in[b:]
             out[p + "dkv.norm"] = self.dkv_norm
         return out
 
@@ -241,12 +318,19 @@ class LatentAttnMixer(_Part):
         proj = _mm(h, self.w_in)
         rows = cache.rows[li if self.owner else s.kv_from]
         if self.owner:
-            seq.latent_kv_store(proj.narrow(1, self.nq + self.nv, self.row),
+            seq.latent_kv_store(proj.narrow(1, self.n0 + self.ng, self.row),
                                 s.kv_rank, self.dkv_norm, model.cfg.norm_eps,
                                 bt.positions, self.inv_freq, rows,
-                                bt.slot_mapping)
-        q = proj.narrow(1, 0, self.nq).unflatten(1, (H, s.dim + s.rot_dim))
-        seq.rope_partial_(q, s.dim, self.inv_freq, bt.positions)
+                                bt.slot_mapping, self.amp, self.interleaved)
+        if self.uq is not None:
+            cq = seq.group_rmsnorm(proj.narrow(1, 0, self.n0), self.dq_norm,
+                                   1, model.cfg.norm_eps, h.dtype)
+            q = _mm(cq, self.uq)
+        else:
+            q = proj.narrow(1, 0, self.nq)
+        q = q.unflatten(1, (H, s.dim + s.rot_dim))
+        seq.rope_partial_(q, s.dim, self.inv_freq, bt.positions, self.amp,
+                          self.interleaved)
         # absorb the key up-projection into the query: (q . W_uk c) =
         # (W_uk^T q) . c, so every head scores against the cached latent
         q_lat = torch.bmm(q[:, :, :s.dim].transpose(0, 1),
@@ -259,7 +343,9 @@ class LatentAttnMixer(_Part):
         o = torch.bmm(o_lat.transpose(0, 1),
                       self.uv.view(H, s.vdim, s.kv_rank).transpose(1, 2))
         o = o.transpose(0, 1).reshape(N, self.nv)
-        o = seq.sigmoid_mul(o, proj.narrow(1, self.nq, self.nv))
+        gate = proj.narrow(1, self.n0, self.ng)
+        o = seq.sigmoid_mul(o, gate) if s.gate == "element" else \
+            seq.sigmoid_mul_heads(o, gate)
         return _mm(o, self.wo)
 
 
@@ -283,6 +369,10 @@ class WindowAttnMixer(_Part):
         if self.b_in is not None:
             self.b_in.zero_()             # the head gate has no bias
         self.sink = z(s.heads, dt=f32) if s.sink else None
+        self.head_bias = z(s.heads, dt=f32) if s.head_bias else None
+        self.v_inv_freq = seq.rope_inv_freq(s.vdim, s.value_rope_base,
+                                            device) \
+            if s.value_rope_base > 0 else None
         self.q_norm = z(self.nq, dt=f32) if s.qk_norm else None
         self.k_norm = z(self.nk, dt=f32) if s.qk_norm else None
         self.wo = z(width, s.heads * s.vdim)
@@ -317,6 +407,8 @@ class WindowAttnMixer(_Part):
                 out[p + "v.b"] = self.b_in[b:b + self.nv]
         if self.sink is not None:
             out[p + "sink"] = self.sink
+        if self.head_bias is not None:
+            out[p + "pb"] = self.head_bias
         return out
 
     def forward(self, h, bt, li, model, cache, states):
@@ -329,14 +421,18 @@ class WindowAttnMixer(_Part):
             proj.narrow(1, b, self.nv) if self.nv else None,
             self.q_norm, self.k_norm, model.cfg.norm_eps, self.inv_freq,
             self.amp, bt.positions, rows, bt.slot_mapping, s.heads,
-            s.kv_heads, s.dim, s.vdim)
+            s.kv_heads, s.dim, s.vdim, head_unit=s.head_unit_norm,
+            v_inv_freq=self.v_inv_freq)
         o = seq.gqa_window_attention(
             q, rows, bt.page_table, bt.seq_of_tok, bt.positions, s.heads,
             s.kv_heads, s.dim, s.vdim, s.window, s.keep_first, self.rel,
             self.dist_bucket,
             proj.narrow(1, b + self.nv, self.ng) if self.ng else None,
             s.scale, h.dtype, tiles=bt.attn_tiles, sink=self.sink,
-            q_temp_coef=s.q_temp_coef, q_temp_every=s.q_temp_every)
+            q_temp_coef=s.q_temp_coef, q_temp_every=s.q_temp_every,
+            softcap=s.softcap, head_bias=self.head_bias,
+            sigmoid_weights=s.weights == "sigmoid",
+            v_inv_freq=self.v_inv_freq)
         return _mm(o, self.wo)
 
 
@@ -447,17 +543,20 @@ class TableMoE(_Part):
 
 
 class RoutedMoE(_Part):
-    """Experts chosen by a softmax router (fp32) with a selection-only
-    correction and group-limited choice; plain experts W_down gelu(W_up h);
-    trailing identity experts return the input; a shared expert runs for
-    every token.  Returns the sublayer output (N, width)."""
+    """Experts chosen by an fp32 router (softmax or per-logit sigmoid
+    scores) with a selection-only correction and group-limited choice;
+    experts W_down gelu(W_up h) or, gated, W_down (silu(W_gate h) * W_up h)
+    with the gate rows stored ahead of the up rows; trailing identity
+    experts return the input; a shared expert runs for every token.
+    Returns the sublayer output (N, width)."""
 
     def __init__(self, spec, width, vocab, device, dtype):
         self.spec = f = spec
         self.E, self.top, self.ff = f.experts, f.top, f.ff
         z = lambda *a, dt=dtype: torch.empty(*a, device=device, dtype=dt)
         f32 = torch.float32
-        self.w_up = z(f.experts, f.ff, width)
+        self.gated = f.expert_act == "silu_gated"
+        self.w_up = z(f.experts, (2 if self.gated else 1) * f.ff, width)
         self.w_down = z(f.experts, width, f.ff)
         self.router = z(f.experts + f.identity, width, dt=f32)
         self.correction = z(f.experts + f.identity, dt=f32)
@@ -467,7 +566,11 @@ class RoutedMoE(_Part):
     def named(self, p):
         out = {p + "router": self.router, p + "correction": self.correction}
         for e in range(self.E):
-            out[f"{p}e{e}.up"] = self.w_up[e]
+            if self.gated:
+                out[f"{p}e{e}.gate"] = self.w_up[e, :self.ff]
+                out[f"{p}e{e}.up"] = self.w_up[e, self.ff:]
+            else:
+                out[f"{p}e{e}.up"] = self.w_up[e]
             out[f"{p}e{e}.down"] = self.w_down[e]
         if self.s_up is not None:
             out[p + "shared.up"] = self.s_up
@@ -496,21 +599,28 @@ class RoutedMoE(_Part):
             if c:
                 step = 64 if c < 512 else 256
                 cp = -(-c // step) * step
-                act = seq.gelu_erf(_mm(xs[o:o + cp], self.w_up[e]))
+                act = self._act(_mm(xs[o:o + cp], self.w_up[e]))
                 ys_sorted[o:o + c] = _mm(act, self.w_down[e])[:c]
                 o += c
         ys = torch.empty_like(ys_sorted)
         ys[order] = ys_sorted           # identity rows stay unread
         return ys
 
+    def _act(self, a):
+        if self.gated:
+            return seq.silu_mul_any(a.narrow(1, 0, self.ff),
+                                    a.narrow(1, self.ff, self.ff))
+        return seq.gelu_erf(a)
+
     def forward(self, h, res, bt):
         f = self.spec
         logits = _mm(h.float(), self.router)
         idx, w = seq.moe_route(logits, self.correction, f.top, f.group_count,
-                               f.group_keep)
+                               f.group_keep, f.router_act, f.group_top)
         if h.shape[0] <= 256 and self.E and \
                 seq.moe_routed_ffn_supported(h, self.top, self.ff):
-            ys = seq.moe_routed_ffn(h, idx, self.w_up, self.w_down)
+            ys = seq.moe_routed_ffn(h, idx, self.w_up, self.w_down,
+                                    self.gated)
         elif self.E:
             ys = self.experts_large(h, idx.long())
         else:
@@ -519,11 +629,11 @@ class RoutedMoE(_Part):
         if self.s_up is not None:
             shared = _mm(seq.gelu_erf(_mm(h, self.s_up)), self.s_down)
         return seq.moe_weighted_combine(ys, idx, w, h, shared, self.E,
-                                        f.weight_eps, h.dtype)
+                                        f.weight_eps, h.dtype, f.route_scale)
 
 
 _MIXERS = {"general_delta": DeltaRuleMixer, "mamba2": SSMMixer,
-           "gla": GLAMixer,
+           "gla": GLAMixer, "rglru": RGLRUMixer,
            "latent_attention": LatentAttnMixer, "attention": WindowAttnMixer}
 _FFS = {"dense": DenseFF, "moe": TableMoE, "routed_moe": RoutedMoE}
 
@@ -614,6 +724,40 @@ class PreNormLayer:
         return out
 
 
+class ParallelLayer:
+    """x += mixer(norm1(x)) + ff(norm2(x)), both norms of the same x
+    (per-channel weights); optionally each sublayer's result passes a
+    sigmoid gate W h + b computed from the sublayer's own input."""
+
+    def __init__(self, cfg: HybridConfig, li: int, device, dtype):
+        L = cfg.layers[li]
+        W = cfg.hidden_size
+        f32 = torch.float32
+        z = lambda *a, dt=dtype: torch.empty(*a, device=device, dtype=dt)
+        self.norm1 = z(W, dt=f32)
+        self.mixer = _MIXERS[L.mixer.kind](L.mixer, W, device, dtype)
+        self.ff = None if L.ff is None else \
+            _FFS[L.ff.kind](L.ff, W, cfg.vocab_size, device, dtype)
+        self.norm2 = z(W, dt=f32) if self.ff is not None else None
+        self.rg1 = self.rg1_b = self.rg2 = self.rg2_b = None
+        if cfg.gated_residual:
+            self.rg1, self.rg1_b = z(W, W), z(W)
+            if self.ff is not None:
+                self.rg2, self.rg2_b = z(W, W), z(W)
+
+    def named(self, p: str) -> Dict[str, torch.Tensor]:
+        out = {p + "norm1": self.norm1}
+        out.update(self.mixer.named(p + "mix."))
+        if self.rg1 is not None:
+            out.update({p + "rg1": self.rg1, p + "rg1.b": self.rg1_b})
+        if self.ff is not None:
+            out[p + "norm2"] = self.norm2
+            out.update(self.ff.named(p + "mlp."))
+            if self.rg2 is not None:
+                out.update({p + "rg2": self.rg2, p + "rg2.b": self.rg2_b})
+        return out
+
+
 class HybridInferenceModel:
     """Weights + packed forward of a hybrid decoder for the rollout engine
     (same weight-update surface as InferenceModel: ``_name_map``,
@@ -640,8 +784,10 @@ class HybridInferenceModel:
                                  "the checkpoint: call resolve_shapes first")
         self.sandwich = cfg.layer_style == "sandwich"
         self.prenorm = cfg.layer_style == "prenorm"
+        self.parallel = cfg.layer_style == "parallel"
         layer_cls = SandwichLayer if self.sandwich else \
-            PreNormLayer if self.prenorm else HybridLayer
+            PreNormLayer if self.prenorm else \
+            ParallelLayer if self.parallel else HybridLayer
         self.layers = [layer_cls(cfg, li, device, dtype)
                        for li in range(cfg.num_hidden_layers)]
         self.runs = cfg.run_order()
@@ -651,7 +797,7 @@ class HybridInferenceModel:
             cfg.vocab_size, cfg.num_hidden_layers * cfg.token_side_dim,
             device=device, dtype=dtype)
         self.final_norm = torch.empty(
-            W if self.sandwich or self.prenorm else 1,
+            W if self.sandwich or self.prenorm or self.parallel else 1,
             device=device, dtype=torch.float32)
         self.lm_head = torch.empty(cfg.vocab_size, W, device=device,
                                    dtype=dtype)
@@ -780,6 +926,15 @@ class HybridInferenceModel:
                 buf.copy_(torch.randn(buf.shape, generator=g) * 0.1)
             elif name == "bigram":
                 buf.copy_(torch.randn(buf.shape, generator=g) * 0.5)
+            elif self.parallel and name.endswith(
+                    ("norm1", "norm2", "final.norm", ".norm")):
+                buf.copy_(1.0 + torch.randn(buf.shape, generator=g) * 0.1)
+            elif self.parallel and name.endswith(".lam"):
+                buf.copy_(torch.randn(buf.shape, generator=g) - 3.0)
+            elif self.parallel and name.endswith(".b"):
+                buf.copy_(torch.randn(buf.shape, generator=g) * 0.2)
+            elif name.endswith("mix.pb"):
+                buf.copy_(torch.randn(buf.shape, generator=g) * 0.5 - 4.0)
             elif self.sandwich and name.endswith(
                     ("norm1", "norm2", "norm1b", "norm2b", "final.norm")):
                 buf.copy_(torch.randn(buf.shape, generator=g) * 0.1)
@@ -827,6 +982,8 @@ class HybridInferenceModel:
             return self._forward_sandwich(bt, cache, states)
         if self.prenorm:
             return self._forward_prenorm(bt, cache, states)
+        if self.parallel:
+            return self._forward_parallel(bt, cache, states)
         cfg, dt = self.cfg, self.dtype
         eps = cfg.norm_eps
         res = self.embed[bt.tokens].float()
@@ -950,9 +1107,58 @@ class HybridInferenceModel:
         settle()
         return res
 
+    def _norms(self, res, y1, g1, y2, g2, w1, w2):
+        """A parallel layer's joint: the pending (gated) sublayer outputs
+        join the fp32 stream and the new row is normed once for each of
+        the next layer's sublayers."""
+        cfg = self.cfg
+        if cfg.norm_kind == "layer":
+            return seq.gated_add_layernorm(res, y1, g1, y2, g2, w1, w2,
+                                           cfg.norm_eps, self.dtype)
+        for y, g in ((y1, g1), (y2, g2)):
+            if y is not None:
+                seq.residual_add_cast(
+                    res, y if g is None else seq.sigmoid_mul(y, g),
+                    torch.float32)
+        if w1 is None:
+            return None, None
+        rms = lambda w: seq.add_rmsnorm_f32res(res, None, w, cfg.norm_eps,
+                                               self.dtype, cfg.norm_offset)
+        return rms(w1), None if w2 is None else rms(w2)
+
+    def _forward_parallel(self, bt: HybridBatch, cache, states):
+        """Layer runs of the parallel style: both sublayers of a run read
+        norms of the same stream; their outputs (and gates) stay pending
+        until the next run's norms, which add them in the same pass over
+        the row."""
+        res = self.embed[bt.tokens].float()
+        y1 = g1 = y2 = g2 = None
+        for ri, li in enumerate(self.runs):
+            L = self.layers[li]
+            h1, h2 = self._norms(res, y1, g1, y2, g2, L.norm1, L.norm2)
+            y1 = L.mixer.forward(h1, bt, ri, self, cache, states)
+            g1 = _mm(h1, L.rg1, L.rg1_b) if L.rg1 is not None else None
+            y2 = g2 = None
+            if L.ff is not None:
+                y2 = L.ff.forward(h2, res, bt)
+                g2 = _mm(h2, L.rg2, L.rg2_b) if L.rg2 is not None else None
+            if self.capture_layers is not None:
+                self._norms(res, y1, g1, y2, g2, None, None)
+                y1 = g1 = y2 = g2 = None
+                self.capture_layers.append(res.clone())
+        self._norms(res, y1, g1, y2, g2, None, None)
+        return res
+
     @torch.no_grad()
     def logits(self, res_rows: torch.Tensor) -> torch.Tensor:
         """Final norm + head on residual rows -> fp32 logits."""
+        if self.cfg.norm_kind == "layer":
+            h = seq.gated_add_layernorm(
+                res_rows.contiguous(), None, None, None, None,
+                self.final_norm, None, self.cfg.norm_eps, self.dtype)[0]
+            return _mm(h, self.lm_head).float() * self.cfg.logit_scale \
+                if self.cfg.logit_scale != 1.0 else \
+                _mm(h, self.lm_head).float()
         h = seq.add_rmsnorm_f32res(res_rows.contiguous(), None,
                                    self.final_norm, self.cfg.norm_eps,
                                    self.dtype, self.cfg.norm_offset)
