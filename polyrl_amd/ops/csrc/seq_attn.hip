@@ -49,7 +49,7 @@ __global__ __launch_bounds__(64) void latent_attn_kernel(
     q[c] = v * scale;
     o[c] = 0.f;
   }
-  float m = sink[h], l = 1.f;
+  float m = sink ? sink[h] : -INFINITY, l = sink ? 1.f : 0.f;
 
   for (int j0 = lo; j0 <= pos; j0 += KB) {
     float kv[KB][NCH], s[KB];
@@ -109,7 +109,8 @@ __global__ __launch_bounds__(64) void latent_attn_kernel(
       (const T*)q_rot.data_ptr(), q_rot.stride(0), q_rot.stride(1),           \
       (const T*)cache.data_ptr(), page_table.data_ptr<int>(),                 \
       (int)page_table.size(1), seq_of_tok.data_ptr<int>(),                    \
-      positions.data_ptr<int>(), sink.data_ptr<float>(), H, R, rd,            \
+      positions.data_ptr<int>(),                                              \
+      has_sink ? sink.data_ptr<float>() : nullptr, H, R, rd,                  \
       (int)cache.size(1), (int)window, (float)scale)
 
 void seq_latent_attention(torch::Tensor out, torch::Tensor q_lat,
@@ -118,7 +119,8 @@ void seq_latent_attention(torch::Tensor out, torch::Tensor q_lat,
                           torch::Tensor positions, int64_t window,
                           torch::Tensor sink, double scale) {
   CHECK_I32(page_table); CHECK_I32(seq_of_tok); CHECK_I32(positions);
-  CHECK_F32(sink);
+  const bool has_sink = sink.defined() && sink.numel() > 0;
+  if (has_sink) CHECK_F32(sink);
   TORCH_CHECK(q_lat.is_cuda() && q_lat.is_contiguous() && q_lat.dim() == 3);
   TORCH_CHECK(q_rot.is_cuda() && q_rot.dim() == 3 && q_rot.stride(2) == 1);
   TORCH_CHECK(out.is_contiguous() && out.sizes() == q_lat.sizes());
@@ -131,7 +133,8 @@ void seq_latent_attention(torch::Tensor out, torch::Tensor q_lat,
   TORCH_CHECK(q_rot.scalar_type() == ty && cache.scalar_type() == ty &&
               out.scalar_type() == ty);
   TORCH_CHECK(page_table.dim() == 2 && seq_of_tok.numel() == N &&
-              positions.numel() == N && sink.numel() == H && window >= 1);
+              positions.numel() == N && (!has_sink || sink.numel() == H) &&
+              window >= 1);
   if (N == 0) return;
   const int nch = (R + rd + 63) / 64;
   TORCH_CHECK(nch <= 12, "latent row above 768 numbers not supported");

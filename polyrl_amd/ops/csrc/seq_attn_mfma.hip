@@ -87,8 +87,8 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const int i = wid * 16 + lhi * 4 + r;
-    m_run[r] = sink[row_head(i)];
-    l_run[r] = 1.f;
+    m_run[r] = sink ? sink[row_head(i)] : -1e30f;   // no sink: nothing yet
+    l_run[r] = sink ? 1.f : 0.f;
     rpos[r] = row_pos(i);
     rok[r] = row_ok(i);
   }
@@ -230,7 +230,8 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
                      page_table.data_ptr<int>(), (int)page_table.size(1),     \
                      seq_of_tok.data_ptr<int>(), positions.data_ptr<int>(),   \
                      tile_n0.data_ptr<int>(), tile_cnt.data_ptr<int>(),       \
-                     sink.data_ptr<float>(), H, (int)rank, rd,                \
+                     has_sink ? sink.data_ptr<float>() : nullptr, H,          \
+                     (int)rank, rd,                                           \
                      (int)cache.size(1), (int)window, (float)scale, (int)mode)
 
 void seq_latent_attention_mfma(torch::Tensor out, torch::Tensor q,
@@ -242,7 +243,8 @@ void seq_latent_attention_mfma(torch::Tensor out, torch::Tensor q,
                                double scale, int64_t mode) {
   CHECK_I32(page_table); CHECK_I32(seq_of_tok); CHECK_I32(positions);
   CHECK_I32(tile_n0); CHECK_I32(tile_cnt);
-  CHECK_F32(sink);
+  const bool has_sink = sink.defined() && sink.numel() > 0;
+  if (has_sink) CHECK_F32(sink);
   TORCH_CHECK(q.is_cuda() && q.is_contiguous() && q.dim() == 3 &&
               q.scalar_type() == torch::kBFloat16);
   const int N = q.size(0), H = q.size(1), row = q.size(2);
@@ -255,7 +257,8 @@ void seq_latent_attention_mfma(torch::Tensor out, torch::Tensor q,
               out.dim() == 3 && out.size(0) == N && out.size(1) == H &&
               out.size(2) == rank);
   TORCH_CHECK(page_table.dim() == 2 && seq_of_tok.numel() == N &&
-              positions.numel() == N && sink.numel() == H && window >= 1);
+              positions.numel() == N && (!has_sink || sink.numel() == H) &&
+              window >= 1);
   TORCH_CHECK(tile_n0.numel() == tile_cnt.numel() && (mode == 0 || mode == 1));
   const int ntiles = tile_n0.numel();
   if (N == 0 || ntiles == 0) return;

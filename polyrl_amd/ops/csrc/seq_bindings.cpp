@@ -24,11 +24,24 @@ void seq_group_rmsnorm(torch::Tensor out, torch::Tensor y,
                        torch::Tensor weight, int64_t groups, double eps,
                        torch::Tensor gate, int64_t gate_act);
 void seq_rope_partial(torch::Tensor q, int64_t offset, torch::Tensor inv_freq,
-                      torch::Tensor positions);
+                      torch::Tensor positions, double amp, bool interleaved);
+void seq_gated_add_layernorm(torch::Tensor out1, torch::Tensor out2,
+                             torch::Tensor res, torch::Tensor y1,
+                             torch::Tensor g1, torch::Tensor y2,
+                             torch::Tensor g2, torch::Tensor w1,
+                             torch::Tensor w2, double eps);
+void seq_sigmoid_mul_heads(torch::Tensor out, torch::Tensor x,
+                           torch::Tensor gate);
+void seq_rglru_scan(torch::Tensor out, torch::Tensor u, torch::Tensor gates,
+                    torch::Tensor gate_bias, torch::Tensor lam,
+                    torch::Tensor y_lin, torch::Tensor state,
+                    torch::Tensor cu_q, torch::Tensor state_slot,
+                    double decay_mult, int64_t max_rows);
 void seq_latent_kv_store(torch::Tensor dkv, int64_t rank, torch::Tensor norm_w,
                          double eps, torch::Tensor positions,
                          torch::Tensor inv_freq, torch::Tensor cache,
-                         torch::Tensor slot_mapping);
+                         torch::Tensor slot_mapping, double amp,
+                         bool interleaved);
 void seq_act_mul(torch::Tensor out, torch::Tensor a, torch::Tensor b,
                  int64_t mode, double p0, double p1, double p2);
 void seq_gelu_mul_rows(torch::Tensor out, torch::Tensor gate,
@@ -69,7 +82,8 @@ void seq_gqa_prepare_store(torch::Tensor q_out, torch::Tensor q,
                            double eps, torch::Tensor inv_freq, double amp,
                            torch::Tensor positions, torch::Tensor cache,
                            torch::Tensor slot_mapping, int64_t H, int64_t G,
-                           int64_t D, int64_t Dv);
+                           int64_t D, int64_t Dv, bool head_unit,
+                           torch::Tensor v_inv_freq);
 void seq_gqa_window_attention(torch::Tensor out, torch::Tensor q,
                               torch::Tensor cache, torch::Tensor page_table,
                               torch::Tensor seq_of_tok,
@@ -78,7 +92,9 @@ void seq_gqa_window_attention(torch::Tensor out, torch::Tensor q,
                               int64_t keep_first, torch::Tensor rel,
                               torch::Tensor dist_bucket, torch::Tensor gate,
                               double scale, torch::Tensor sink,
-                              double q_temp_coef, int64_t q_temp_every);
+                              double q_temp_coef, int64_t q_temp_every,
+                              double softcap, torch::Tensor head_bias,
+                              bool sigmoid_weights, torch::Tensor v_inv_freq);
 void seq_gqa_window_attention_mfma(
     torch::Tensor out, torch::Tensor q, torch::Tensor tile_n0,
     torch::Tensor tile_cnt, torch::Tensor cache, torch::Tensor page_table,
@@ -86,16 +102,18 @@ void seq_gqa_window_attention_mfma(
     int64_t D, int64_t Dv, int64_t window, int64_t keep_first,
     torch::Tensor rel, torch::Tensor dist_bucket, torch::Tensor gate,
     double scale, torch::Tensor sink, double q_temp_coef,
-    int64_t q_temp_every);
+    int64_t q_temp_every, double softcap, torch::Tensor head_bias,
+    bool sigmoid_weights, torch::Tensor v_inv_freq);
 void seq_moe_route(torch::Tensor idx, torch::Tensor w, torch::Tensor logits,
-                   torch::Tensor correction, int64_t groups, int64_t keep);
+                   torch::Tensor correction, int64_t groups, int64_t keep,
+                   int64_t act, int64_t group_top);
 void seq_moe_routed_ffn(torch::Tensor y, torch::Tensor act, torch::Tensor h,
                         torch::Tensor idx, torch::Tensor w_up,
-                        torch::Tensor w_down);
+                        torch::Tensor w_down, bool gated);
 void seq_moe_weighted_combine(torch::Tensor out, torch::Tensor ys,
                               torch::Tensor idx, torch::Tensor w,
                               torch::Tensor h, torch::Tensor shared,
-                              int64_t E, double weight_eps);
+                              int64_t E, double weight_eps, double scale);
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("seq_gqa_prepare_store", &seq_gqa_prepare_store,
@@ -105,9 +123,15 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("seq_gqa_window_attention_mfma", &seq_gqa_window_attention_mfma,
         "grouped-query window attention on the matrix cores (bf16)");
   m.def("seq_moe_route", &seq_moe_route,
-        "softmax router with correction and group-limited top-k");
+        "softmax / sigmoid router with correction and group-limited top-k");
   m.def("seq_moe_routed_ffn", &seq_moe_routed_ffn,
-        "router-chosen plain experts for decode-sized bf16 batches");
+        "router-chosen plain or gated experts for decode-sized bf16 batches");
+  m.def("seq_gated_add_layernorm", &seq_gated_add_layernorm,
+        "fp32 residual += gated branches, layer norm once per weight vector");
+  m.def("seq_sigmoid_mul_heads", &seq_sigmoid_mul_heads,
+        "rows times one sigmoid gate per head");
+  m.def("seq_rglru_scan", &seq_rglru_scan,
+        "real-gated linear recurrence (fp32 state, in place)");
   m.def("seq_moe_weighted_combine", &seq_moe_weighted_combine,
         "weighted sum of chosen experts, identity experts and shared");
   m.def("seq_embed_compose", &seq_embed_compose,
@@ -121,7 +145,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("seq_group_rmsnorm", &seq_group_rmsnorm,
         "grouped RMS norm with optional sigmoid / SiLU gate");
   m.def("seq_rope_partial", &seq_rope_partial,
-        "rotate-half RoPE on a slice of each head, in place");
+        "RoPE (halves or interleaved pairs) on a slice of each head, in place");
   m.def("seq_latent_kv_store", &seq_latent_kv_store,
         "norm + rotate + write latent cache rows");
   m.def("seq_act_mul", &seq_act_mul, "silu*b / sigmoid*b / tanh / gelu / clamped gated unit");

@@ -22,6 +22,17 @@
 // sink, the running sum at one), and a query temperature that multiplies
 // the score scale of the row at position p by
 // 1 + coef * ln(floor((p + 1) / every) + 1).
+//
+// Further options of the writer (gqa_prepare_heads_kernel, one wave per
+// head): every query and key head is divided by its own root mean square
+// AFTER the rotation (no weight), and every value head is rotated over all
+// its entries by its position (pairs (m, m + Dv/2)) before it is cached.
+// Further options of the attention kernels: scores capped as
+// cap * tanh(score / cap), a number per head added to the capped score, and
+// weights sigmoid(score) per visible key with no normalisation over the
+// keys (the running maximum and sum are then unused).  The head sums can be
+// written as fp32 to a separate buffer for a pass that turns them back by
+// the row's position.
 #include <torch/extension.h>
 #include <ATen/hip/HIPContext.h>
 
@@ -85,13 +96,80 @@ __global__ __launch_bounds__(256) void gqa_prepare_kernel(
   for (int i = threadIdx.x; i < nv; i += 256) crow[nk + i] = vr[i];
 }
 
+// One wave per head of a token (H query heads, G key heads, G value heads;
+// four waves a block take them in turn).  Query / key heads: rotate the
+// first 2*half entries, then (unit) divide the head by its root mean square;
+// the statistics are taken of the rotated numbers, which are computed again
+// for the store (nothing is rounded in between).  Value heads: rotate all Dv
+// entries in halves with their own frequencies, or copy.
+template <typename T>
+__global__ __launch_bounds__(256) void gqa_prepare_heads_kernel(
+    T* __restrict__ q_out, const T* __restrict__ q, long ldq,
+    const T* __restrict__ k, long ldk, const T* __restrict__ v, long ldv,
+    float eps, const float* __restrict__ inv_freq, int half, float amp,
+    const float* __restrict__ v_freq, const int* __restrict__ positions,
+    T* __restrict__ cache, const int* __restrict__ slot_mapping, int H, int G,
+    int D, int Dv, bool unit) {
+  const long n = blockIdx.x;
+  const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const float pos = (float)positions[n];
+  T* crow = cache + (long)slot_mapping[n] * (G * (D + Dv));
+  for (int hu = wid; hu < H + 2 * G; hu += 4) {
+    const T* src;
+    T* dst;
+    int dim, hf;
+    const float* fr;
+    float am;
+    bool un;
+    if (hu < H) {
+      src = q + n * ldq + (long)hu * D;
+      dst = q_out + (n * H + hu) * D;
+      dim = D; hf = half; fr = inv_freq; am = amp; un = unit;
+    } else if (hu < H + G) {
+      src = k + n * ldk + (long)(hu - H) * D;
+      dst = crow + (hu - H) * D;
+      dim = D; hf = half; fr = inv_freq; am = amp; un = unit;
+    } else {
+      src = v + n * ldv + (long)(hu - H - G) * Dv;
+      dst = crow + G * D + (hu - H - G) * Dv;
+      dim = Dv; hf = v_freq ? Dv / 2 : 0; fr = v_freq; am = 1.f; un = false;
+    }
+    float inv = 1.f;
+    if (un) {
+      float ss = 0.f;
+      for (int i = lane; i < hf; i += 64) {
+        const float ang = pos * fr[i];
+        const float c = cosf(ang) * am, s = sinf(ang) * am;
+        const float a = ldf(src + i), b = ldf(src + i + hf);
+        const float x = a * c - b * s, y = b * c + a * s;
+        ss += x * x + y * y;
+      }
+      for (int i = 2 * hf + lane; i < dim; i += 64) {
+        const float a = ldf(src + i);
+        ss += a * a;
+      }
+      inv = rsqrtf(wave_reduce_sum(ss) / dim + eps);
+    }
+    for (int i = lane; i < hf; i += 64) {
+      const float ang = pos * fr[i];
+      const float c = cosf(ang) * am, s = sinf(ang) * am;
+      const float a = ldf(src + i), b = ldf(src + i + hf);
+      stf(dst + i, (a * c - b * s) * inv);
+      stf(dst + i + hf, (b * c + a * s) * inv);
+    }
+    for (int i = 2 * hf + lane; i < dim; i += 64)
+      stf(dst + i, ldf(src + i) * inv);
+  }
+}
+
 void seq_gqa_prepare_store(torch::Tensor q_out, torch::Tensor q,
                            torch::Tensor k, torch::Tensor v,
                            torch::Tensor q_norm, torch::Tensor k_norm,
                            double eps, torch::Tensor inv_freq, double amp,
                            torch::Tensor positions, torch::Tensor cache,
                            torch::Tensor slot_mapping, int64_t H, int64_t G,
-                           int64_t D, int64_t Dv) {
+                           int64_t D, int64_t Dv, bool head_unit,
+                           torch::Tensor v_inv_freq) {
   CHECK_ROWS(q);
   CHECK_ROWS(k);
   CHECK_I32(positions);
@@ -124,6 +202,27 @@ void seq_gqa_prepare_store(torch::Tensor q_out, torch::Tensor q,
   TORCH_CHECK(positions.numel() == N && slot_mapping.numel() == N);
   if (N == 0) return;
   auto stream = at::hip::getCurrentHIPStream();
+  const bool v_rot = v_inv_freq.defined() && v_inv_freq.numel() > 0;
+  if (head_unit || v_rot) {
+    TORCH_CHECK(!has_norm, "whole-row and per-head norms do not combine");
+    TORCH_CHECK(has_v, "the per-head writer needs a value projection");
+    if (v_rot) {
+      CHECK_F32(v_inv_freq);
+      TORCH_CHECK(Dv % 2 == 0 && v_inv_freq.numel() == Dv / 2,
+                  "one frequency per value pair");
+    }
+    SEQ_DISPATCH_T(ty, { hipLaunchKernelGGL((gqa_prepare_heads_kernel<T>), dim3(N), dim3(256), 0, stream,
+        (T*)q_out.data_ptr(), (const T*)q.data_ptr(), q.stride(0),
+        (const T*)k.data_ptr(), k.stride(0), (const T*)v.data_ptr(),
+        v.stride(0), (float)eps,
+        half ? inv_freq.data_ptr<float>() : nullptr, half, (float)amp,
+        v_rot ? v_inv_freq.data_ptr<float>() : nullptr,
+        positions.data_ptr<int>(), (T*)cache.data_ptr(),
+        slot_mapping.data_ptr<int>(), (int)H, (int)G, (int)D, (int)Dv,
+        head_unit); });
+    HIP_CHECK_KERNEL();
+    return;
+  }
   SEQ_DISPATCH_T(ty, { hipLaunchKernelGGL((gqa_prepare_kernel<T>), dim3(N), dim3(256), 0, stream,
       (T*)q_out.data_ptr(), (const T*)q.data_ptr(), q.stride(0),
       (const T*)k.data_ptr(), k.stride(0),
@@ -218,7 +317,8 @@ __global__ __launch_bounds__(256) void gqa_attn_kernel(
     const T* __restrict__ gate, long ldg,  // (N, H) view or null
     int H, int G, int D, int Dv, int page_size, int window, int keep,
     float scale, bool vec, int lpr, const float* __restrict__ sink,
-    float qt_coef, int qt_every) {
+    float qt_coef, int qt_every, float cap, const float* __restrict__ hbias,
+    bool sigm, float* __restrict__ out32) {
   constexpr int EPL = Vec16<T>::N;
   __shared__ float q_sh[4][NCH * 64];
   __shared__ float p_sh[4][64];
@@ -249,6 +349,7 @@ __global__ __launch_bounds__(256) void gqa_attn_kernel(
 #pragma unroll
   for (int k = 0; k < EPL; ++k) ov[k] = 0.f;
   float m = sink ? sink[h] : -INFINITY, l = sink ? 1.f : 0.f;
+  const float hb = hbias ? hbias[h] : 0.f;
   const int kgrp = lpr ? lane / lpr : 0;          // key of an iteration
   const int dcol = lpr ? (lane % lpr) * EPL : 0;  // first value entry
   const int kper = lpr ? 64 / lpr : 1;            // keys per iteration
@@ -261,12 +362,20 @@ __global__ __launch_bounds__(256) void gqa_attn_kernel(
     const int slot = ptab[j / page_size] * page_size + j % page_size;
     float s = dot_row<T>(cache + (long)slot * row + koff, qs, D, vec) * scale;
     if (rel) s += rel[(long)dist_bucket[pos - j] * H + h];
+    if (cap > 0.f) s = cap * tanhf(s / cap);
+    s += hb;
     if (!valid) s = -INFINITY;
-    const float mn = fmaxf(m, wave_reduce_max(s));
-    const float p = valid ? expf(s - mn) : 0.f;
-    const float corr = expf(m - mn);
-    l = l * corr + wave_reduce_sum(p);
-    m = mn;
+    float p, corr;
+    if (sigm) {
+      p = valid ? sigmoidf_acc(s) : 0.f;
+      corr = 1.f;
+    } else {
+      const float mn = fmaxf(m, wave_reduce_max(s));
+      p = valid ? expf(s - mn) : 0.f;
+      corr = expf(m - mn);
+      l = l * corr + wave_reduce_sum(p);
+      m = mn;
+    }
     ps[lane] = p;
     ss[lane] = slot;
     const int cntk = total - base < 64 ? total - base : 64;
@@ -299,8 +408,8 @@ __global__ __launch_bounds__(256) void gqa_attn_kernel(
       }
     }
   }
-  float inv = 1.f / l;
-  if (gate) inv *= sigmoidf_acc(ldf(gate + n * ldg + h));
+  float inv = sigm ? 1.f : 1.f / l;
+  if (gate && !out32) inv *= sigmoidf_acc(ldf(gate + n * ldg + h));
   if (lpr) {
 #pragma unroll
     for (int k = 0; k < EPL; ++k)
@@ -308,17 +417,26 @@ __global__ __launch_bounds__(256) void gqa_attn_kernel(
         ov[k] += __shfl_xor(ov[k], off, WAVE_SIZE);
     if (lane < lpr) {
 #pragma unroll
-      for (int k = 0; k < EPL; ++k)
-        stf(out + (n * H + h) * Dv + dcol + k, ov[k] * inv);
+      for (int k = 0; k < EPL; ++k) {
+        if (out32) out32[(n * H + h) * Dv + dcol + k] = ov[k] * inv;
+        else stf(out + (n * H + h) * Dv + dcol + k, ov[k] * inv);
+      }
     }
     return;
   }
 #pragma unroll
   for (int c = 0; c < NCH; ++c) {
     const int d = lane + 64 * c;
-    if (d < Dv) stf(out + (n * H + h) * Dv + d, o[c] * inv);
+    if (d < Dv) {
+      if (out32) out32[(n * H + h) * Dv + d] = o[c] * inv;
+      else stf(out + (n * H + h) * Dv + d, o[c] * inv);
+    }
   }
 }
+
+void seq_rotate_back_heads(torch::Tensor out, torch::Tensor x,
+                           torch::Tensor inv_freq, torch::Tensor positions,
+                           torch::Tensor gate, int64_t H);
 
 // shared argument checks of both attention entry points
 void gqa_attention_check(torch::Tensor out, torch::Tensor q,
@@ -374,7 +492,9 @@ void gqa_attention_check(torch::Tensor out, torch::Tensor q,
       has_gate ? gate.stride(0) : 0, (int)H, (int)G, (int)D, (int)Dv,         \
       (int)cache.size(1), (int)window, (int)keep_first, (float)scale, vec,     \
       lpr, has_sink ? sink.data_ptr<float>() : nullptr, (float)q_temp_coef,   \
-      (int)q_temp_every)
+      (int)q_temp_every, (float)softcap,                                      \
+      has_hb ? head_bias.data_ptr<float>() : nullptr, sigmoid_weights,        \
+      o32)
 
 void seq_gqa_window_attention(torch::Tensor out, torch::Tensor q,
                               torch::Tensor cache, torch::Tensor page_table,
@@ -384,12 +504,30 @@ void seq_gqa_window_attention(torch::Tensor out, torch::Tensor q,
                               int64_t keep_first, torch::Tensor rel,
                               torch::Tensor dist_bucket, torch::Tensor gate,
                               double scale, torch::Tensor sink,
-                              double q_temp_coef, int64_t q_temp_every) {
+                              double q_temp_coef, int64_t q_temp_every,
+                              double softcap, torch::Tensor head_bias,
+                              bool sigmoid_weights, torch::Tensor v_inv_freq) {
   gqa_attention_check(out, q, cache, page_table, seq_of_tok, positions, H, G,
                       D, Dv, window, keep_first, rel, dist_bucket, gate, sink,
                       q_temp_every);
   const int N = q.size(0);
   if (N == 0) return;
+  const bool has_hb = head_bias.defined() && head_bias.numel() > 0;
+  if (has_hb) {
+    CHECK_F32(head_bias);
+    TORCH_CHECK(head_bias.numel() == H, "one bias per query head");
+  }
+  TORCH_CHECK(!sigmoid_weights || !(sink.defined() && sink.numel() > 0),
+              "a sink needs softmax weights");
+  // rotated values: the head sums leave as fp32 and a second pass turns
+  // them back by the row's position (and applies the gate)
+  const bool v_rot = v_inv_freq.defined() && v_inv_freq.numel() > 0;
+  torch::Tensor sums;
+  float* o32 = nullptr;
+  if (v_rot) {
+    sums = torch::empty({q.size(0), H * Dv}, q.options().dtype(torch::kFloat32));
+    o32 = sums.data_ptr<float>();
+  }
   const bool has_sink = sink.defined() && sink.numel() > 0;
   const bool has_rel = rel.defined() && rel.numel() > 0;
   const bool has_gate = gate.defined() && gate.numel() > 0;
@@ -411,4 +549,5 @@ void seq_gqa_window_attention(torch::Tensor out, torch::Tensor q,
     }
   });
   HIP_CHECK_KERNEL();
+  if (v_rot) seq_rotate_back_heads(out, sums, v_inv_freq, positions, gate, H);
 }

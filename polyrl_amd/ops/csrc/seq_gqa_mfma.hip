@@ -14,6 +14,10 @@
 // LDS), the online softmax and the sigmoid head gate are fp32; so are the
 // optional sink (the running maximum starts at the head's sink, the running
 // sum at one) and the per-row query temperature folded into the score scale.
+// Options: scores capped as cap * tanh(score / cap), a number per head added
+// to the capped score, and weights sigmoid(score) per live key without any
+// normalisation over keys (no running maximum, no rescaling); head sums as
+// fp32 into a separate buffer for the pass that turns rotated values back.
 // The next tiles are fetched into registers while the current ones are
 // multiplied.
 // K-tile bytes are XOR-swizzled by row inside each 64-byte chunk.
@@ -53,7 +57,8 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(
     const int* __restrict__ dist_bucket,
     const bf16_t* __restrict__ gate, long ldg, int H, int G, int D, int Dv,
     int page_size, int window, int keep, float scale,
-    const float* __restrict__ sink, float qt_coef, int qt_every) {
+    const float* __restrict__ sink, float qt_coef, int qt_every, float cap,
+    const float* __restrict__ hbias, bool sigm, float* __restrict__ out32) {
   constexpr int DKP = KS * 32;           // padded head size in LDS
   constexpr int NVT = KS * 2;            // 16-wide output tiles
   __shared__ __attribute__((aligned(16))) bf16_t Ks[GKV * DKP];
@@ -104,6 +109,8 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(
                         : __builtin_bit_cast(bf16x8_t, zi);
     }
   }
+  const float hb = hbias ? hbias[h] : 0.f;
+  const float inv_cap = cap > 0.f ? 1.f / cap : 0.f;
   float m_run[4], l_run[4], rscale[4];
   int rpos[4];
   bool rok[4];
@@ -196,7 +203,16 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(
                           (dist < window || j < keep);
         float sv = c[nt][r] * rscale[r];
         if (rel && live) sv += rel_s[dist_bucket[dist]];
+        if (cap > 0.f) sv = cap * tanhf(sv * inv_cap);
+        sv += hb;
         s[nt] = live ? sv : -1e30f;
+      }
+      if (sigm) {
+        alpha[r] = 1.f;
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+          p[nt][r] = s[nt] > -1e29f ? sigmoidf_acc(s[nt]) : 0.f;
+        continue;
       }
       float rm = fmaxf(s[0], s[1]);
 #pragma unroll
@@ -215,10 +231,12 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(
       for (int off = 1; off < 16; off <<= 1) rs += __shfl_xor(rs, off, 64);
       l_run[r] = l_run[r] * alpha[r] + rs;
     }
+    if (!sigm) {
 #pragma unroll
-    for (int nt = 0; nt < NVT; ++nt)
+      for (int nt = 0; nt < NVT; ++nt)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) o_acc[nt][r] *= alpha[r];
+        for (int r = 0; r < 4; ++r) o_acc[nt][r] *= alpha[r];
+    }
 
     // ---- P: C layout -> A layout through a wave-private LDS tile --------
     bf16_t* ps = Ps[wid];
@@ -253,13 +271,17 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(
     const int i = wid * 16 + lhi * 4 + r;
     if (!rok[r]) continue;
     const long tok = n0 + i;
-    float inv = 1.f / l_run[r];
-    if (gate) inv *= sigmoidf_acc(bf2f(gate[tok * ldg + h]));
+    float inv = sigm ? 1.f : 1.f / l_run[r];
+    if (gate && !out32) inv *= sigmoidf_acc(bf2f(gate[tok * ldg + h]));
     bf16_t* op = out + (tok * H + h) * Dv;
+    float* op32 = out32 ? out32 + (tok * H + h) * Dv : nullptr;
 #pragma unroll
     for (int nt = 0; nt < NVT; ++nt) {
       const int d = nt * 16 + l15;
-      if (d < Dv) op[d] = f2bf(o_acc[nt][r] * inv);
+      if (d < Dv) {
+        if (op32) op32[d] = o_acc[nt][r] * inv;
+        else op[d] = f2bf(o_acc[nt][r] * inv);
+      }
     }
   }
 }
@@ -280,7 +302,12 @@ void seq_gqa_window_attention(torch::Tensor out, torch::Tensor q,
                               int64_t keep_first, torch::Tensor rel,
                               torch::Tensor dist_bucket, torch::Tensor gate,
                               double scale, torch::Tensor sink,
-                              double q_temp_coef, int64_t q_temp_every);
+                              double q_temp_coef, int64_t q_temp_every,
+                              double softcap, torch::Tensor head_bias,
+                              bool sigmoid_weights, torch::Tensor v_inv_freq);
+void seq_rotate_back_heads(torch::Tensor out, torch::Tensor x,
+                           torch::Tensor inv_freq, torch::Tensor positions,
+                           torch::Tensor gate, int64_t H);
 
 #define GQA_MFMA_LAUNCH(KSV)                                                  \
   hipLaunchKernelGGL((gqa_attn_mfma_kernel<KSV>), grid, dim3(256), 0, stream, \
@@ -296,7 +323,8 @@ void seq_gqa_window_attention(torch::Tensor out, torch::Tensor q,
       has_gate ? gate.stride(0) : 0, (int)H, (int)G, (int)D, (int)Dv,         \
       (int)cache.size(1), (int)window, (int)keep_first, (float)scale,         \
       has_sink ? sink.data_ptr<float>() : nullptr, (float)q_temp_coef,        \
-      (int)q_temp_every)
+      (int)q_temp_every, (float)softcap,                                      \
+      has_hb ? head_bias.data_ptr<float>() : nullptr, sigmoid_weights, o32)
 
 void seq_gqa_window_attention_mfma(
     torch::Tensor out, torch::Tensor q, torch::Tensor tile_n0,
@@ -305,7 +333,8 @@ void seq_gqa_window_attention_mfma(
     int64_t D, int64_t Dv, int64_t window, int64_t keep_first,
     torch::Tensor rel, torch::Tensor dist_bucket, torch::Tensor gate,
     double scale, torch::Tensor sink, double q_temp_coef,
-    int64_t q_temp_every) {
+    int64_t q_temp_every, double softcap, torch::Tensor head_bias,
+    bool sigmoid_weights, torch::Tensor v_inv_freq) {
   gqa_attention_check(out, q, cache, page_table, seq_of_tok, positions, H, G,
                       D, Dv, window, keep_first, rel, dist_bucket, gate, sink,
                       q_temp_every);
@@ -320,11 +349,25 @@ void seq_gqa_window_attention_mfma(
     seq_gqa_window_attention(out, q, cache, page_table, seq_of_tok, positions,
                              H, G, D, Dv, window, keep_first, rel,
                              dist_bucket, gate, scale, sink, q_temp_coef,
-                             q_temp_every);
+                             q_temp_every, softcap, head_bias,
+                             sigmoid_weights, v_inv_freq);
     return;
   }
   const int ntiles = tile_n0.numel();
   if (q.size(0) == 0 || ntiles == 0) return;
+  const bool has_hb = head_bias.defined() && head_bias.numel() > 0;
+  if (has_hb) {
+    CHECK_F32(head_bias);
+    TORCH_CHECK(head_bias.numel() == H, "one bias per query head");
+  }
+  TORCH_CHECK(!sigmoid_weights || !has_sink, "a sink needs softmax weights");
+  const bool v_rot = v_inv_freq.defined() && v_inv_freq.numel() > 0;
+  torch::Tensor sums;
+  float* o32 = nullptr;
+  if (v_rot) {
+    sums = torch::empty({q.size(0), H * Dv}, q.options().dtype(torch::kFloat32));
+    o32 = sums.data_ptr<float>();
+  }
   // (tile, kv head) units in rounds of one per XCD, H/G heads per unit
   const long units = (long)ntiles * G;
   const long rounds = (units + GQA_XCDS - 1) / GQA_XCDS;
@@ -338,4 +381,5 @@ void seq_gqa_window_attention_mfma(
     default: GQA_MFMA_LAUNCH(4); break;
   }
   HIP_CHECK_KERNEL();
+  if (v_rot) seq_rotate_back_heads(out, sums, v_inv_freq, positions, gate, H);
 }

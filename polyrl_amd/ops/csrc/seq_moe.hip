@@ -138,11 +138,13 @@ void seq_moe_table_ffn(torch::Tensor y, torch::Tensor act, torch::Tensor h,
   HIP_CHECK_KERNEL();
 }
 
-// y (B*top, width) = router-chosen plain experts on h (B, width); fills
-// ``act`` (B*top, ff) on the way.  Rows of identity experts stay unwritten.
+// y (B*top, width) = router-chosen experts on h (B, width), plain
+// (gelu(W_up h), w_up (E, ff, W)) or gated (silu(W_gate h) * W_up h, w_up
+// (E, 2*ff, W) with the gate rows first); fills ``act`` (B*top, ff) on the
+// way.  Rows of identity experts stay unwritten.
 void seq_moe_routed_ffn(torch::Tensor y, torch::Tensor act, torch::Tensor h,
                         torch::Tensor idx, torch::Tensor w_up,
-                        torch::Tensor w_down) {
+                        torch::Tensor w_down, bool gated) {
   CHECK_I32(idx);
   TORCH_CHECK(h.is_cuda() && h.dim() == 2 && h.stride(1) == 1 &&
               h.scalar_type() == torch::kBFloat16);
@@ -153,7 +155,8 @@ void seq_moe_routed_ffn(torch::Tensor y, torch::Tensor act, torch::Tensor h,
   const int B = h.size(0), W = h.size(1);
   TORCH_CHECK(idx.dim() == 2 && idx.size(0) == B);
   const int top = idx.size(1);
-  const int E = w_up.size(0), ff = w_up.size(1);
+  const int E = w_up.size(0), ff = w_up.size(1) / (gated ? 2 : 1);
+  TORCH_CHECK(!gated || w_up.size(1) % 2 == 0);
   TORCH_CHECK(w_up.size(2) == W && w_down.size(0) == E &&
               w_down.size(1) == W && w_down.size(2) == ff);
   TORCH_CHECK(W % 32 == 0 && ff % 32 == 0 && h.stride(0) % 8 == 0,
@@ -165,12 +168,20 @@ void seq_moe_routed_ffn(torch::Tensor y, torch::Tensor act, torch::Tensor h,
               y.size(0) == (long)B * top && y.size(1) == W);
   if (B == 0 || E == 0) return;
   auto stream = at::hip::getCurrentHIPStream();
-  hipLaunchKernelGGL((moe_table_gemm_kernel<2>), dim3((ff + 63) / 64, E),
-                     dim3(256), 0, stream, (bf16_t*)act.data_ptr(),
-                     (const bf16_t*)h.data_ptr(), h.stride(0),
-                     (const long*)nullptr, (const int*)nullptr,
-                     idx.data_ptr<int>(), (const bf16_t*)w_up.data_ptr(), B,
-                     top, W, ff);
+  if (gated)
+    hipLaunchKernelGGL((moe_table_gemm_kernel<1>), dim3((ff + 63) / 64, E),
+                       dim3(256), 0, stream, (bf16_t*)act.data_ptr(),
+                       (const bf16_t*)h.data_ptr(), h.stride(0),
+                       (const long*)nullptr, (const int*)nullptr,
+                       idx.data_ptr<int>(), (const bf16_t*)w_up.data_ptr(), B,
+                       top, W, ff);
+  else
+    hipLaunchKernelGGL((moe_table_gemm_kernel<2>), dim3((ff + 63) / 64, E),
+                       dim3(256), 0, stream, (bf16_t*)act.data_ptr(),
+                       (const bf16_t*)h.data_ptr(), h.stride(0),
+                       (const long*)nullptr, (const int*)nullptr,
+                       idx.data_ptr<int>(), (const bf16_t*)w_up.data_ptr(), B,
+                       top, W, ff);
   hipLaunchKernelGGL((moe_table_gemm_kernel<0>), dim3((W + 63) / 64, E),
                      dim3(256), 0, stream, (bf16_t*)y.data_ptr(),
                      (const bf16_t*)act.data_ptr(), (long)ff,
@@ -181,12 +192,14 @@ void seq_moe_routed_ffn(torch::Tensor y, torch::Tensor act, torch::Tensor h,
 }
 
 // ------------------------------------------------------------------ router
-// One wave per token, four tokens a block.  s = softmax(logits) over all E router outputs;
+// One wave per token, four tokens a block.  s = softmax(logits) over all E
+// router outputs, or (act 1) the logistic function of every logit;
 // choice = s + correction; experts form ``groups`` equal groups of
-// neighbours and only the ``keep`` groups with the largest best choice stay
-// eligible (the others count as minus infinity); the ``top`` largest
-// eligible choices win, ties to the lower index.  Writes the indices and the
-// UNcorrected s at them.
+// neighbours, a group's score is the sum of its ``gtop`` largest choices,
+// and only the ``keep`` groups with the largest score stay eligible (the
+// others count as minus infinity); the ``top`` largest eligible choices
+// win, ties to the lower index.  Writes the indices and the UNcorrected s
+// at them.
 constexpr int ROUTE_MAX_E = 512;
 
 DEV_INLINE void wave_argmax(float& v, int& i) {
@@ -205,7 +218,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(
     int* __restrict__ idx, float* __restrict__ wout,
     const float* __restrict__ logits, long ldl,
     const float* __restrict__ correction, long N, int E, int top, int groups,
-    int keep) {
+    int keep, int act, int gtop) {
   __shared__ float s_sh[4][ROUTE_MAX_E], c_sh[4][ROUTE_MAX_E];
   __shared__ float g_sh[4][ROUTE_MAX_E];
   const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -216,28 +229,54 @@ __global__ __launch_bounds__(256) void moe_route_kernel(
   float* c = c_sh[wid];
   float* gb = g_sh[wid];
   const float* z = logits + n * ldl;
-  float mx = -INFINITY;
-  for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
-  mx = wave_reduce_max(mx);
-  float sum = 0.f;
-  for (int e = lane; e < E; e += 64) {
-    const float p = expf(z[e] - mx);
-    s[e] = p;
-    sum += p;
-  }
-  sum = wave_reduce_sum(sum);
-  const float inv = 1.f / sum;
-  for (int e = lane; e < E; e += 64) {
-    const float p = s[e] * inv;
-    s[e] = p;
-    c[e] = p + correction[e];
+  if (act == 1) {
+    for (int e = lane; e < E; e += 64) {
+      const float p = sigmoidf_acc(z[e]);
+      s[e] = p;
+      c[e] = p + correction[e];
+    }
+  } else {
+    float mx = -INFINITY;
+    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
+    mx = wave_reduce_max(mx);
+    float sum = 0.f;
+    for (int e = lane; e < E; e += 64) {
+      const float p = expf(z[e] - mx);
+      s[e] = p;
+      sum += p;
+    }
+    sum = wave_reduce_sum(sum);
+    const float inv = 1.f / sum;
+    for (int e = lane; e < E; e += 64) {
+      const float p = s[e] * inv;
+      s[e] = p;
+      c[e] = p + correction[e];
+    }
   }
   __syncthreads();
   if (groups > 1) {
     const int per = E / groups;
     for (int g = lane; g < groups; g += 64) {
-      float b = -INFINITY;
-      for (int e = g * per; e < (g + 1) * per; ++e) b = fmaxf(b, c[e]);
+      // sum of the gtop largest choices of the group: pick them one by one,
+      // each below the last pick in (value, -index) order
+      float b = 0.f, lv = INFINITY;
+      int li = -1;
+      const int take = gtop < per ? gtop : per;
+      for (int r = 0; r < take; ++r) {
+        float bv = -INFINITY;
+        int bi = -1;
+        for (int e = g * per; e < (g + 1) * per; ++e) {
+          const float v = c[e];
+          const bool below = v < lv || (v == lv && e > li);
+          if (below && (bi < 0 || v > bv)) {
+            bv = v;
+            bi = e;
+          }
+        }
+        b += bv;
+        lv = bv;
+        li = bi;
+      }
       gb[g] = b;
     }
     __syncthreads();
@@ -284,7 +323,8 @@ __global__ __launch_bounds__(256) void moe_route_kernel(
 }
 
 void seq_moe_route(torch::Tensor idx, torch::Tensor w, torch::Tensor logits,
-                   torch::Tensor correction, int64_t groups, int64_t keep) {
+                   torch::Tensor correction, int64_t groups, int64_t keep,
+                   int64_t act, int64_t group_top) {
   CHECK_I32(idx);
   CHECK_F32(w);
   CHECK_F32(correction);
@@ -297,24 +337,25 @@ void seq_moe_route(torch::Tensor idx, torch::Tensor w, torch::Tensor logits,
   TORCH_CHECK(E >= 1 && E <= ROUTE_MAX_E, "router outputs above 512");
   TORCH_CHECK(correction.numel() == E && top >= 1 && top <= E);
   TORCH_CHECK(groups >= 1 && E % groups == 0 && keep >= 1 && keep <= groups);
+  TORCH_CHECK((act == 0 || act == 1) && group_top >= 1);
   if (N == 0) return;
   auto stream = at::hip::getCurrentHIPStream();
   hipLaunchKernelGGL(moe_route_kernel, dim3((N + 3) / 4), dim3(256), 0, stream,
                      idx.data_ptr<int>(), w.data_ptr<float>(),
                      logits.data_ptr<float>(), logits.stride(0),
                      correction.data_ptr<float>(), N, E, top, (int)groups,
-                     (int)keep);
+                     (int)keep, (int)act, (int)group_top);
   HIP_CHECK_KERNEL();
 }
 
 // out[n, d] = sum_k w'[n,k] * (idx[n,k] < E ? ys[n*top+k, d] : h[n, d])
-//             (+ shared[n, d]),  w' = w / (sum_k w + weight_eps)
+//             (+ shared[n, d]),  w' = scale * w / (sum_k w + weight_eps)
 template <typename T>
 __global__ void moe_weighted_combine_kernel(
     T* __restrict__ out, const T* __restrict__ ys, const int* __restrict__ idx,
     const float* __restrict__ w, const T* __restrict__ h, long ldh,
     const T* __restrict__ shared, long lds_, int top, int E, float weight_eps,
-    long rows, int D) {
+    long rows, int D, float scale) {
   long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
   const long stride = (long)gridDim.x * blockDim.x;
   for (; i < rows * D; i += stride) {
@@ -322,7 +363,7 @@ __global__ void moe_weighted_combine_kernel(
     const int d = i % D;
     float wsum = 0.f;
     for (int k = 0; k < top; ++k) wsum += w[n * top + k];
-    const float inv = 1.f / (wsum + weight_eps);
+    const float inv = scale / (wsum + weight_eps);
     float acc = 0.f;
     for (int k = 0; k < top; ++k) {
       const float v = idx[n * top + k] < E ? ldf(ys + (n * top + k) * D + d)
@@ -337,7 +378,7 @@ __global__ void moe_weighted_combine_kernel(
 void seq_moe_weighted_combine(torch::Tensor out, torch::Tensor ys,
                               torch::Tensor idx, torch::Tensor w,
                               torch::Tensor h, torch::Tensor shared,
-                              int64_t E, double weight_eps) {
+                              int64_t E, double weight_eps, double scale) {
   CHECK_I32(idx);
   CHECK_F32(w);
   CHECK_ROWS(h);
@@ -365,6 +406,6 @@ void seq_moe_weighted_combine(torch::Tensor out, torch::Tensor ys,
       w.data_ptr<float>(), (const T*)h.data_ptr(), h.stride(0),
       has_shared ? (const T*)shared.data_ptr() : nullptr,
       has_shared ? shared.stride(0) : 0, top, (int)E, (float)weight_eps, N,
-      D); });
+      D, (float)scale); });
   HIP_CHECK_KERNEL();
 }

@@ -389,28 +389,30 @@ void seq_group_rmsnorm(torch::Tensor out, torch::Tensor y,
 }
 
 // ---------------------------------------------------- partial rotary (q)
-// q (N, H, Dh) with token stride ldn: rotate the pair (off+i, off+i+half)
-// by angle fp32(pos) * inv_freq[i].
+// q (N, H, Dh) with token stride ldn: rotate the pair (off+i, off+i+half),
+// or (off+2i, off+2i+1) when the pairs are interleaved, by angle
+// fp32(pos) * inv_freq[i]; cos and sin are multiplied by amp.
 template <typename T>
 __global__ void rope_partial_kernel(T* __restrict__ q, long ldn, int H, int Dh,
                                     int off, const float* __restrict__ inv_freq,
                                     int half, const int* __restrict__ pos,
-                                    long total) {
+                                    long total, float amp, bool inter) {
   long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total) return;
   const int i = idx % half;
   const int h = (idx / half) % H;
   const long n = idx / ((long)half * H);
   const float ang = (float)pos[n] * inv_freq[i];
-  const float c = cosf(ang), s = sinf(ang);
-  T* p = q + n * ldn + (long)h * Dh + off + i;
-  const float a = ldf(p), b = ldf(p + half);
+  const float c = cosf(ang) * amp, s = sinf(ang) * amp;
+  T* p = q + n * ldn + (long)h * Dh + off + (inter ? 2 * i : i);
+  const int step = inter ? 1 : half;
+  const float a = ldf(p), b = ldf(p + step);
   stf(p, a * c - b * s);
-  stf(p + half, b * c + a * s);
+  stf(p + step, b * c + a * s);
 }
 
 void seq_rope_partial(torch::Tensor q, int64_t offset, torch::Tensor inv_freq,
-                      torch::Tensor positions) {
+                      torch::Tensor positions, double amp, bool interleaved) {
   CHECK_F32(inv_freq);
   CHECK_I32(positions);
   TORCH_CHECK(q.is_cuda() && q.dim() == 3 && q.stride(2) == 1 &&
@@ -424,19 +426,20 @@ void seq_rope_partial(torch::Tensor q, int64_t offset, torch::Tensor inv_freq,
   SEQ_DISPATCH_T(q.scalar_type(), { hipLaunchKernelGGL((rope_partial_kernel<T>), dim3((total + 255) / 256), dim3(256), 0, stream, 
       (T*)q.data_ptr(), q.stride(0), (int)q.size(1), (int)q.size(2),
       (int)offset, inv_freq.data_ptr<float>(), half,
-      positions.data_ptr<int>(), total); });
+      positions.data_ptr<int>(), total, (float)amp, interleaved); });
   HIP_CHECK_KERNEL();
 }
 
 // ------------------------------------------------------ latent cache store
 // one wave per token: RMS-norm the latent (first R columns) times norm_w,
-// rotate the first 2*half columns of the key part, write the cache row.
+// rotate the first 2*half columns of the key part (pairs in halves or
+// interleaved, cos/sin times amp), write the cache row.
 template <typename T>
 __global__ __launch_bounds__(64) void latent_store_kernel(
     const T* __restrict__ dkv, long ld, int R, int rd,
     const float* __restrict__ norm_w, float eps, const int* __restrict__ pos,
     const float* __restrict__ inv_freq, int half, T* __restrict__ cache,
-    const int* __restrict__ slot_mapping) {
+    const int* __restrict__ slot_mapping, float amp, bool inter) {
   const long n = blockIdx.x;
   const int lane = threadIdx.x;
   const int slot = slot_mapping[n];
@@ -454,10 +457,11 @@ __global__ __launch_bounds__(64) void latent_store_kernel(
   const float p = (float)pos[n];
   for (int i = lane; i < half; i += 64) {
     const float ang = p * inv_freq[i];
-    const float c = cosf(ang), s = sinf(ang);
-    const float a = ldf(src + R + i), b = ldf(src + R + i + half);
-    stf(dst + R + i, a * c - b * s);
-    stf(dst + R + i + half, b * c + a * s);
+    const float c = cosf(ang) * amp, s = sinf(ang) * amp;
+    const int ia = inter ? 2 * i : i, ib = inter ? 2 * i + 1 : i + half;
+    const float a = ldf(src + R + ia), b = ldf(src + R + ib);
+    stf(dst + R + ia, a * c - b * s);
+    stf(dst + R + ib, b * c + a * s);
   }
   for (int i = 2 * half + lane; i < rd; i += 64) stf(dst + R + i, ldf(src + R + i));
 }
@@ -465,7 +469,8 @@ __global__ __launch_bounds__(64) void latent_store_kernel(
 void seq_latent_kv_store(torch::Tensor dkv, int64_t rank, torch::Tensor norm_w,
                          double eps, torch::Tensor positions,
                          torch::Tensor inv_freq, torch::Tensor cache,
-                         torch::Tensor slot_mapping) {
+                         torch::Tensor slot_mapping, double amp,
+                         bool interleaved) {
   CHECK_ROWS(dkv);
   CHECK_F32(norm_w);
   CHECK_F32(inv_freq);
@@ -484,7 +489,7 @@ void seq_latent_kv_store(torch::Tensor dkv, int64_t rank, torch::Tensor norm_w,
       (const T*)dkv.data_ptr(), dkv.stride(0), (int)rank, (int)(row - rank),
       norm_w.data_ptr<float>(), (float)eps, positions.data_ptr<int>(),
       inv_freq.data_ptr<float>(), half, (T*)cache.data_ptr(),
-      slot_mapping.data_ptr<int>()); });
+      slot_mapping.data_ptr<int>(), (float)amp, interleaved); });
   HIP_CHECK_KERNEL();
 }
 
@@ -608,5 +613,199 @@ void seq_moe_combine(torch::Tensor res, torch::Tensor y, torch::Tensor inv,
   SEQ_DISPATCH_T(y.scalar_type(), { hipLaunchKernelGGL((moe_combine_kernel<T>), dim3((n + 255) / 256), dim3(256), 0, stream, 
       res.data_ptr<float>(), (const T*)y.data_ptr(), inv.data_ptr<int>(),
       (int)inv.size(1), (float)scale, res.size(0), (int)res.size(1)); });
+  HIP_CHECK_KERNEL();
+}
+
+// ------------------------------------------- gated joint + shared layer norm
+// One block per row.  res (fp32) += y1 * sigmoid(g1) [+ y2 * sigmoid(g2)]
+// (a missing gate: plain add; a missing y1: no add), then the layer norm of
+// the new row, (x - mean) * rsqrt(var + eps), is written once per weight
+// vector: out1 = unit * w1, out2 = unit * w2.  Two sublayers that read the
+// same stream share the statistics, so their norms cost one pass.  The
+// variance is the mean of the squared deviations (second pass over values
+// the thread itself wrote).
+template <typename T>
+__global__ __launch_bounds__(256) void gated_add_layernorm_kernel(
+    T* __restrict__ out1, T* __restrict__ out2, float* __restrict__ res,
+    const T* __restrict__ y1, long ld1, const T* __restrict__ g1, long ldg1,
+    const T* __restrict__ y2, long ld2, const T* __restrict__ g2, long ldg2,
+    const float* __restrict__ w1, const float* __restrict__ w2, int D,
+    float eps) {
+  __shared__ float red[8], red2[8];
+  const long row = blockIdx.x;
+  float* rr = res + row * D;
+  float sum = 0.f;
+  for (int i = threadIdx.x; i < D; i += 256) {
+    float f = rr[i];
+    if (y1) {
+      float a = ldf(y1 + row * ld1 + i);
+      if (g1) a *= sigmoidf_acc(ldf(g1 + row * ldg1 + i));
+      if (y2) {
+        float b = ldf(y2 + row * ld2 + i);
+        if (g2) b *= sigmoidf_acc(ldf(g2 + row * ldg2 + i));
+        a += b;
+      }
+      f += a;
+      rr[i] = f;
+    }
+    sum += f;
+  }
+  if (!out1) return;
+  const float mean = block_reduce_sum<4>(sum, red) / D;
+  float sq = 0.f;
+  for (int i = threadIdx.x; i < D; i += 256) {
+    const float d = rr[i] - mean;          // own writes: same thread, same i
+    sq += d * d;
+  }
+  const float inv = rsqrtf(block_reduce_sum<4>(sq, red2) / D + eps);
+  for (int i = threadIdx.x; i < D; i += 256) {
+    const float u = (rr[i] - mean) * inv;
+    stf(out1 + row * D + i, u * w1[i]);
+    if (out2) stf(out2 + row * D + i, u * w2[i]);
+  }
+}
+
+void seq_gated_add_layernorm(torch::Tensor out1, torch::Tensor out2,
+                             torch::Tensor res, torch::Tensor y1,
+                             torch::Tensor g1, torch::Tensor y2,
+                             torch::Tensor g2, torch::Tensor w1,
+                             torch::Tensor w2, double eps) {
+  CHECK_F32(res);
+  TORCH_CHECK(res.dim() == 2);
+  const long rows = res.size(0);
+  const int D = res.size(1);
+  if (rows == 0) return;
+  auto has = [](const torch::Tensor& t) { return t.defined() && t.numel() > 0; };
+  const bool h1 = has(out1), h2 = has(out2);
+  TORCH_CHECK(h1 || !h2, "a second norm needs the first");
+  TORCH_CHECK(has(y1) || (!has(g1) && !has(y2) && !has(g2)));
+  TORCH_CHECK(has(y2) || !has(g2));
+  TORCH_CHECK(h1 || has(y1), "nothing to do");
+  auto ty = h1 ? out1.scalar_type() : y1.scalar_type();
+  for (const torch::Tensor* t : {&y1, &g1, &y2, &g2}) {
+    if (!has(*t)) continue;
+    TORCH_CHECK(t->is_cuda() && t->dim() == 2 && t->stride(1) == 1 &&
+                t->size(0) == rows && t->size(1) == D &&
+                t->scalar_type() == ty, "branch rows / dtype");
+  }
+  for (const torch::Tensor* t : {&out1, &out2}) {
+    if (!has(*t)) continue;
+    TORCH_CHECK(t->is_cuda() && t->is_contiguous() &&
+                t->numel() == res.numel() && t->scalar_type() == ty);
+  }
+  if (h1) { CHECK_F32(w1); TORCH_CHECK(w1.numel() == D); }
+  if (h2) { CHECK_F32(w2); TORCH_CHECK(w2.numel() == D); }
+  auto stream = at::hip::getCurrentHIPStream();
+  SEQ_DISPATCH_T(ty, {
+    auto p = [&](const torch::Tensor& t) {
+      return has(t) ? (const T*)t.data_ptr() : (const T*)nullptr; };
+    auto ld = [&](const torch::Tensor& t) { return has(t) ? t.stride(0) : 0L; };
+    hipLaunchKernelGGL((gated_add_layernorm_kernel<T>), dim3(rows), dim3(256),
+        0, stream, h1 ? (T*)out1.data_ptr() : nullptr,
+        h2 ? (T*)out2.data_ptr() : nullptr, res.data_ptr<float>(), p(y1),
+        ld(y1), p(g1), ld(g1), p(y2), ld(y2), p(g2), ld(g2),
+        h1 ? w1.data_ptr<float>() : nullptr,
+        h2 ? w2.data_ptr<float>() : nullptr, D, (float)eps);
+  });
+  HIP_CHECK_KERNEL();
+}
+
+// ---------------------------------------------- per-head sigmoid gate
+// out[n, h*Dv + d] = x[n, h*Dv + d] * sigmoid(gate[n, h])
+template <typename T>
+__global__ void sigmoid_mul_heads_kernel(T* __restrict__ out,
+                                         const T* __restrict__ x, long ldx,
+                                         const T* __restrict__ gate, long ldg,
+                                         int H, int Dv, long total) {
+  long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const int hd = H * Dv;
+  const long n = i / hd;
+  const int c = i % hd;
+  stf(out + i, ldf(x + n * ldx + c) *
+                   sigmoidf_acc(ldf(gate + n * ldg + c / Dv)));
+}
+
+void seq_sigmoid_mul_heads(torch::Tensor out, torch::Tensor x,
+                           torch::Tensor gate) {
+  CHECK_ROWS(x);
+  CHECK_ROWS(gate);
+  const long N = x.size(0);
+  const int H = gate.size(1);
+  TORCH_CHECK(gate.size(0) == N && H > 0 && x.size(1) % H == 0);
+  TORCH_CHECK(out.is_cuda() && out.is_contiguous() &&
+              out.sizes() == x.sizes() &&
+              out.scalar_type() == x.scalar_type() &&
+              gate.scalar_type() == x.scalar_type());
+  const long total = N * x.size(1);
+  if (total == 0) return;
+  auto stream = at::hip::getCurrentHIPStream();
+  SEQ_DISPATCH_T(x.scalar_type(), {
+    hipLaunchKernelGGL((sigmoid_mul_heads_kernel<T>),
+        dim3((total + 255) / 256), dim3(256), 0, stream, (T*)out.data_ptr(),
+        (const T*)x.data_ptr(), x.stride(0), (const T*)gate.data_ptr(),
+        gate.stride(0), H, (int)(x.size(1) / H), total);
+  });
+  HIP_CHECK_KERNEL();
+}
+
+// ----------------------------------- turn every head's row back (fp32 in)
+// x (N, H*Dv) fp32: head sums over values that were rotated by their own
+// positions.  Pair (m, m + Dv/2) of every head is rotated by
+// -fp32(pos) * inv_freq[m]; then the optional per-head sigmoid gate; the
+// result is rounded once, to T.
+template <typename T>
+__global__ void rotate_back_heads_kernel(T* __restrict__ out,
+                                         const float* __restrict__ x,
+                                         const float* __restrict__ inv_freq,
+                                         const int* __restrict__ pos,
+                                         const T* __restrict__ gate, long ldg,
+                                         int H, int Dv, long total) {
+  long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const int half = Dv / 2;
+  const int m = i % half;
+  const int h = (i / half) % H;
+  const long n = i / ((long)half * H);
+  const float ang = (float)pos[n] * inv_freq[m];
+  const float c = cosf(ang), s = sinf(ang);
+  const long at = (n * H + h) * Dv + m;
+  const float a = x[at], b = x[at + half];
+  float g = 1.f;
+  if (gate) g = sigmoidf_acc(ldf(gate + n * ldg + h));
+  stf(out + at, (a * c + b * s) * g);
+  stf(out + at + half, (b * c - a * s) * g);
+}
+
+void seq_rotate_back_heads(torch::Tensor out, torch::Tensor x,
+                           torch::Tensor inv_freq, torch::Tensor positions,
+                           torch::Tensor gate, int64_t H) {
+  CHECK_F32(x);
+  CHECK_F32(inv_freq);
+  CHECK_I32(positions);
+  TORCH_CHECK(x.dim() == 2 && H > 0 && x.size(1) % H == 0);
+  const long N = x.size(0);
+  const int Dv = x.size(1) / H;
+  TORCH_CHECK(Dv % 2 == 0 && inv_freq.numel() == Dv / 2 &&
+              positions.numel() == N);
+  TORCH_CHECK(out.is_cuda() && out.is_contiguous() &&
+              out.sizes() == x.sizes());
+  const bool has_gate = gate.defined() && gate.numel() > 0;
+  if (has_gate) {
+    CHECK_ROWS(gate);
+    TORCH_CHECK(gate.size(0) == N && gate.size(1) == H &&
+                gate.scalar_type() == out.scalar_type());
+  }
+  const long total = N * H * (Dv / 2);
+  if (total == 0) return;
+  auto stream = at::hip::getCurrentHIPStream();
+  SEQ_DISPATCH_T(out.scalar_type(), {
+    hipLaunchKernelGGL((rotate_back_heads_kernel<T>),
+        dim3((total + 255) / 256), dim3(256), 0, stream, (T*)out.data_ptr(),
+        x.data_ptr<float>(), inv_freq.data_ptr<float>(),
+        positions.data_ptr<int>(),
+        has_gate ? (const T*)gate.data_ptr() : nullptr,
+        has_gate ? gate.stride(0) : 0, (int)H, Dv, total);
+  });
   HIP_CHECK_KERNEL();
 }

@@ -535,6 +535,8 @@ def gated_add_layernorm(res, y1, g1, y2, g2, w1, w2, eps: float, out_dtype):
     Returns (h1, h2) in out_dtype; h2 is None without w2, both without
     w1."""
     if res.is_cuda:
+        if y1 is None and w1 is None:
+            return None, None
         e = torch.Tensor()
         new = lambda: torch.empty(res.shape, dtype=out_dtype,
                                   device=res.device)
@@ -549,7 +551,7 @@ def gated_add_layernorm(res, y1, g1, y2, g2, w1, w2, eps: float, out_dtype):
 
 
 def rglru_scan(u, gates, gate_bias, lam, y_lin, state, cu_q, state_slot,
-               decay_mult: float, out_dtype) -> torch.Tensor:
+               decay_mult: float, out_dtype, max_rows: int = 0) -> torch.Tensor:
     """Real-gated linear recurrence over packed rows; ``state`` (slots, C)
     fp32 in place.  Channels form B equal blocks of bw; ``gates`` (B, N,
     2*bw) fp32 holds the block-diagonal products for the decay gate (first
@@ -557,12 +559,13 @@ def rglru_scan(u, gates, gate_bias, lam, y_lin, state, cu_q, state_slot,
     channel: r = sigmoid(.), i = sigmoid(.), log a = -decay_mult * r *
     softplus(lam), S <- a S + sqrt(1 - a^2) * i * u; returns
     S * gelu_tanh(y_lin) (N, C).  ``u`` and ``y_lin`` may be column
-    slices."""
+    slices.  ``max_rows`` bounds the rows of one sequence (0 = unknown):
+    long portions are cut into segments that run in parallel."""
     if u.is_cuda:
         out = torch.empty(u.shape, dtype=out_dtype, device=u.device)
         if u.shape[0]:
             _ext().seq_rglru_scan(out, u, gates, gate_bias, lam, y_lin, state,
-                                  cu_q, state_slot, decay_mult)
+                                  cu_q, state_slot, decay_mult, max_rows)
         return out
     return R.rglru_scan(u, gates, gate_bias, lam, y_lin, state, cu_q,
                         state_slot, decay_mult, out_dtype)

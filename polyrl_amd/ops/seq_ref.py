@@ -469,7 +469,7 @@ def rglru_scan(u, gates, gate_bias, lam, y_lin, state, cu_q, state_slot,
     log_a = -decay_mult * r * torch.nn.functional.softplus(
         lam.float(), threshold=1e9)
     a = torch.exp(log_a)
-    drive = torch.sqrt(1.0 - a * a) * i * u.float()
+    drive = torch.sqrt(-torch.expm1(2.0 * log_a)) * i * u.float()
     y = gelu_tanh(y_lin.float())
     out = torch.empty(N, C, dtype=torch.float32, device=u.device)
     cu = cu_q.tolist()

@@ -848,7 +848,8 @@ class Engine:
             slot_mapping=i32(maps) if singles else torch.cat(maps).to(dev),
             page_table=torch.from_numpy(ptab).to(dev),
             attn_tiles=ops.seq.attention_tiles(
-                [len(it[2]) for it in items], dev)), cu
+                [len(it[2]) for it in items], dev),
+            max_q=max((len(it[2]) for it in items), default=0)), cu
 
     def _run_mixed(self, prefill_reqs, prefill_lens, decode_reqs):
         """One forward over prompt portions and single decode tokens
@@ -920,7 +921,7 @@ class Engine:
                 cu_q=torch.arange(B + 1, dtype=i32, device=dev),
                 state_slot=z(B), slot_mapping=z(B),
                 page_table=z(B, max(self.kv.num_pages, 1)),
-                attn_tiles=(z(B), z(B), 1))
+                attn_tiles=(z(B), z(B), 1), max_q=1)
             st = {"bt": sb}
             self._load_static(sb, bt)
             saved = {k: t.clone() for k, t in self.states.tensors.items()}

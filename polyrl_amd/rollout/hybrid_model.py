@@ -40,6 +40,7 @@ class HybridBatch:
     slot_mapping: torch.Tensor    # (N,) cache row of each token
     page_table: torch.Tensor      # (B, max_pages)
     attn_tiles: Optional[tuple] = None   # ops.seq.attention_tiles(lens)
+    max_q: int = 0                # rows of the longest portion (0 = unknown)
 
 
 _TUNED = False
@@ -214,7 +215,8 @@ class RGLRUMixer(_Part):
                           self.w_gate.transpose(1, 2))      # (B, N, 2bw)
         y = seq.rglru_scan(u, gates, self.b_gate, self.lam,
                            proj.narrow(1, 0, C), states.tensors[(li, "S")],
-                           bt.cu_q, bt.state_slot, s.decay_mult, h.dtype)
+                           bt.cu_q, bt.state_slot, s.decay_mult, h.dtype,
+                           max_rows=bt.max_q)
         return _mm(y, self.wo)
 
 
@@ -323,8 +325,9 @@ class LatentAttnMixer(_Part):
                                 bt.positions, self.inv_freq, rows,
                                 bt.slot_mapping, self.amp, self.interleaved)
         if self.uq is not None:
-            cq = seq.group_rmsnorm(proj.narrow(1, 0, self.n0), self.dq_norm,
-                                   1, model.cfg.norm_eps, h.dtype)
+            cq = seq.group_rmsnorm(
+                proj.narrow(1, 0, self.n0).float().contiguous(),
+                self.dq_norm, 1, model.cfg.norm_eps, h.dtype)
             q = _mm(cq, self.uq)
         else:
             q = proj.narrow(1, 0, self.nq)

@@ -28,7 +28,8 @@ CORE = ("bindings.cpp", "gemm_tuned.cpp", "elementwise.hip",
         "kv_cache.hip", "attention_decode.hip", "attention_prefill.hip",
         "attention_backward.hip", "attention_backward_v3.hip")
 SEQ = ("seq_bindings.cpp", "seq_ops.hip", "seq_scan.hip", "seq_attn.hip",
-       "seq_moe.hip", "seq_attn_mfma.hip", "seq_gqa.hip", "seq_gqa_mfma.hip")
+       "seq_moe.hip", "seq_attn_mfma.hip", "seq_gqa.hip", "seq_gqa_mfma.hip",
+       "seq_lru.hip")
 
 # scalar fp32 code only: the compiler must not form packed-fp32 VALU ops
 HIPCC_FLAGS = ["-O3", "-std=c++17", "--offload-arch=gfx950",
