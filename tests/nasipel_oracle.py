@@ -108,16 +108,17 @@ def sigmoid_attention(W, p, m, h, eps):
           for t in range(T)]
     vs = [[turn(v[t, g], t, fv, 1.0, False) for g in range(G)]
           for t in range(T)]
+    K = [torch.stack([ks[t][g] for t in range(T)]) for g in range(G)]
+    V = [torch.stack([vs[t][g] for t in range(T)]) for g in range(G)]
     out = torch.zeros(T, H * Dv, dtype=DT)
     for i in range(T):
         for a in range(H):
             g = a // (H // G)
-            acc = torch.zeros(Dv, dtype=DT)
-            for j in range(i + 1):
-                s = float(qs[i][a] @ ks[j][g]) * float(m["scale"])
-                if cap > 0:
-                    s = cap * math.tanh(s / cap)
-                acc = acc + vs[j][g] / (1.0 + math.exp(-(s + float(pb[a]))))
+            s = (K[g][:i + 1] @ qs[i][a]) * float(m["scale"])   # keys 0..i
+            if cap > 0:
+                s = cap * torch.tanh(s / cap)
+            w = sigmoid(s + pb[a])                  # one weight per key
+            acc = (w.unsqueeze(1) * V[g][:i + 1]).sum(0)
             out[i, a * Dv:(a + 1) * Dv] = turn(acc, -i, fv, 1.0, False)
     return out @ _f(W[p + "o"]).t()
 
@@ -138,14 +139,14 @@ def latent_attention(W, p, m, h, eps):
     c = unit_rms(dkv[:, :R], eps) * _f(W[p + "dkv.norm"])
     kn = (c @ _f(W[p + "uk"]).t()).view(T, H, D)
     vv = (c @ _f(W[p + "uv"]).t()).view(T, H, Dv)
-    kr = [turn(dkv[t, R:], t, f, amp, True) for t in range(T)]
+    kr = torch.stack([turn(dkv[t, R:], t, f, amp, True) for t in range(T)])
     gate = sigmoid(h @ _f(W[p + "g"]).t())                # (T, H)
     out = torch.zeros(T, H * Dv, dtype=DT)
     for i in range(T):
         for a in range(H):
             qr = turn(q[i, a, D:], i, f, amp, True)
-            s = torch.stack([(q[i, a, :D] @ kn[j, a] + qr @ kr[j])
-                             * float(m["scale"]) for j in range(i + 1)])
+            s = (kn[:i + 1, a] @ q[i, a, :D] + kr[:i + 1] @ qr) \
+                * float(m["scale"])
             w = torch.softmax(s, 0)
             out[i, a * Dv:(a + 1) * Dv] = (w.unsqueeze(1) * vv[:i + 1, a]
                                            ).sum(0) * gate[i, a]
@@ -264,3 +265,69 @@ def forward(cfg, W, tokens, collect=None):
         if collect is not None:
             collect.append(x.clone())
     return layer_norm(x, W["final.norm"], eps) @ _f(W["head"]).t()
+
+
+# --------------------------------------------------------------- weights
+def random_weights(cfg, seed=0):
+    """name -> tensor for a config; values are bf16-representable so every
+    engine dtype loads them exactly."""
+    g = torch.Generator().manual_seed(seed)
+    Wd, V = int(cfg["width"]), int(cfg["vocab"])
+
+    def rnd(*shape, std=1.0, mean=0.0):
+        return (torch.randn(*shape, generator=g) * std + mean) \
+            .bfloat16().float()
+
+    def lin(o, i, gain=1.0):
+        return rnd(o, i, std=gain / math.sqrt(i))
+    W = {"embed": rnd(V, Wd), "final.norm": rnd(Wd, std=0.1, mean=1.0),
+         "head": lin(V, Wd)}
+    for li, L in enumerate(cfg["layers"]):
+        p, m, kind = f"l{li}.", L["mixer"], L["type"]
+        W[p + "norm1"] = rnd(Wd, std=0.1, mean=1.0)
+        W[p + "rg1"], W[p + "rg1.b"] = lin(Wd, Wd), rnd(Wd, std=0.5)
+        q = p + "mix."
+        if kind == "rglru":
+            C, B, taps = int(m["width"]), int(m["blocks"]), int(m["conv"])
+            bw = C // B
+            W[q + "y"], W[q + "y.b"] = lin(C, Wd), rnd(C, std=0.3)
+            W[q + "x"], W[q + "x.b"] = lin(C, Wd), rnd(C, std=0.3)
+            W[q + "conv"] = rnd(C, taps, std=0.5)
+            W[q + "conv.b"] = rnd(C, std=0.2)
+            for n in ("ra", "ri"):
+                W[q + n] = rnd(B, bw, bw, std=1.0 / math.sqrt(bw))
+                W[q + n + ".b"] = rnd(B, bw, std=0.5)
+            W[q + "lam"] = rnd(C, std=1.0, mean=-2.0)
+            W[q + "o"] = lin(Wd, C)
+        elif kind == "attention":
+            H, G = int(m["heads"]), int(m["kv_heads"])
+            D, Dv = int(m["dim"]), int(m["vdim"])
+            W[q + "q"], W[q + "k"] = lin(H * D, Wd), lin(G * D, Wd)
+            W[q + "v"] = lin(G * Dv, Wd)
+            W[q + "pb"] = rnd(H, std=0.5, mean=-2.0)
+            W[q + "o"] = lin(Wd, H * Dv)
+        else:
+            H, D, Dr = int(m["heads"]), int(m["dim"]), int(m["rot_dim"])
+            Dv, R, Rq = int(m["vdim"]), int(m["kv_rank"]), int(m["q_rank"])
+            W[q + "dq"] = lin(Rq, Wd)
+            W[q + "dq.norm"] = rnd(Rq, std=0.1, mean=1.0)
+            W[q + "uq"] = lin(H * (D + Dr), Rq, gain=2.0)
+            W[q + "dkv"] = lin(R + Dr, Wd)
+            W[q + "dkv.norm"] = rnd(R, std=0.1, mean=1.0)
+            W[q + "uk"] = lin(H * D, R, gain=2.0)
+            W[q + "uv"] = lin(H * Dv, R)
+            W[q + "g"] = lin(H, Wd, gain=2.0)
+            W[q + "o"] = lin(Wd, H * Dv)
+        f = L.get("mlp")
+        if f is None:
+            continue
+        W[p + "norm2"] = rnd(Wd, std=0.1, mean=1.0)
+        W[p + "rg2"], W[p + "rg2.b"] = lin(Wd, Wd), rnd(Wd, std=0.5)
+        E, ff = int(f["router"]["experts"]), int(f["expert"]["ff"])
+        for e in range(E):
+            W[f"{p}mlp.e{e}.gate"] = lin(ff, Wd)
+            W[f"{p}mlp.e{e}.up"] = lin(ff, Wd)
+            W[f"{p}mlp.e{e}.down"] = lin(Wd, ff)
+        W[p + "mlp.router"] = lin(E, Wd, gain=3.0)
+        W[p + "mlp.correction"] = rnd(E, std=0.1)
+    return W

@@ -553,3 +553,190 @@ def test_causal_attention_with_sink_and_temperature(dt, H, G, D, Dv, coef,
             0, None, None, None, scale, dt, tiles=tl, sink=g(sink),
             q_temp_coef=coef, q_temp_every=every)
         torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dt))
+
+
+# ------------------------------------------- gated joints, recurrence, options
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("D", [48, 200, 2048])
+def test_gated_add_layernorm(dt, D):
+    N = 9
+    res = rnd(N, D) + 0.7                    # a mean that matters
+    big = rnd(N, 4 * D + 8, dt=dt)
+    y1, g1 = big[:, 3:3 + D], big[:, 3 + D:3 + 2 * D]
+    y2, g2 = big[:, 5 + 2 * D:5 + 3 * D], big[:, 5 + 3 * D:5 + 4 * D]
+    w1, w2 = rnd(D) + 1, rnd(D) + 1
+    g = lambda t: None if t is None else t.to(DEV)
+    bg = big.to(DEV)
+    dv = lambda t: None if t is None else \
+        bg[:, t.storage_offset():t.storage_offset() + D]
+    for a1, b1, a2, b2, wa, wb in [(y1, g1, y2, g2, w1, w2),
+                                   (y1, g1, None, None, w1, None),
+                                   (y1, None, y2, g2, w1, w2),
+                                   (None, None, None, None, w1, w2),
+                                   (y1, g1, y2, None, None, None)]:
+        r0, r1 = res.clone(), res.clone().to(DEV)
+        want = R.gated_add_layernorm(r0, a1, b1, a2, b2, wa, wb, 1e-5, dt)
+        got = seq.gated_add_layernorm(r1, dv(a1), dv(b1), dv(a2), dv(b2),
+                                      g(wa), g(wb), 1e-5, dt)
+        torch.testing.assert_close(r1.cpu(), r0, rtol=1e-5, atol=1e-5)
+        for x, y in zip(got, want):
+            assert (x is None) == (y is None)
+            if x is not None:
+                torch.testing.assert_close(x.cpu().float(), y.float(),
+                                           **tol(dt))
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("B,bw,lens,max_rows", [
+    (5, 8, [5, 1, 2, 9], 9), (1, 300, [3, 1], 0), (7, 1, [2, 2, 1, 7], 7),
+    (3, 24, [300, 1, 70], 300), (2, 160, [257, 256], 0)])
+def test_rglru_scan(dt, B, bw, lens, max_rows):
+    C = B * bw
+    slots = [3, 0, 5, 1][:len(lens)]
+    bt = batch(lens, slots)
+    N = sum(lens)
+    big = rnd(N, 2 * C + 11, dt=dt)
+    u, y = big[:, 4:4 + C], big[:, 9 + C:9 + 2 * C]
+    gates, gb = rnd(B, N, 2 * bw), rnd(B, 2 * bw)
+    lam = rnd(C) - 3.0
+    st0 = rnd(6, C)
+    s0, s1 = st0.clone(), st0.clone().to(DEV)
+    cu, sl, _ = bt["cpu"]
+    want = R.rglru_scan(u, gates, gb, lam, y, s0, cu, sl, 8.0, dt)
+    cu, sl, _ = bt[DEV]
+    bg = big.to(DEV)
+    got = seq.rglru_scan(bg[:, 4:4 + C], gates.to(DEV), gb.to(DEV),
+                         lam.to(DEV), bg[:, 9 + C:9 + 2 * C], s1, cu, sl, 8.0,
+                         dt, max_rows=max_rows)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dt))
+    torch.testing.assert_close(s1.cpu(), s0, rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("inter", [False, True])
+def test_rotation_pairs_and_amplitude(dt, inter):
+    lens, starts, page = [5, 1, 3], [0, 37, 6], 4
+    R_, rd, H, D = 24, 12, 3, 10
+    cache, ptab, pos, sot, slot = _paged(lens, starts, page, R_ + rd, dt)
+    N = sum(lens)
+    inv = torch.rand(4)
+    q = rnd(N, H, D + rd, dt=dt)
+    want = R.rope_partial_(q.clone(), D, inv, pos, 1.13, inter)
+    got = seq.rope_partial_(q.clone().to(DEV), D, inv.to(DEV), pos.to(DEV),
+                            1.13, inter)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dt))
+    dkv, w = rnd(N, R_ + rd + 3, dt=dt), rnd(R_) + 1
+    c0, c1 = cache.clone(), cache.clone().to(DEV)
+    R.latent_kv_store(dkv[:, :R_ + rd], R_, w, 1e-5, pos, inv, c0, slot, 1.13,
+                      inter)
+    seq.latent_kv_store(dkv.to(DEV)[:, :R_ + rd], R_, w.to(DEV), 1e-5,
+                        pos.to(DEV), inv.to(DEV), c1, slot.to(DEV), 1.13,
+                        inter)
+    torch.testing.assert_close(c1.cpu().float(), c0.float(), **tol(dt))
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("H,G,D,Dv,half,cap,lens,starts", [
+    (4, 2, 24, 24, 4, 5.0, [5, 1, 3], [0, 37, 6]),
+    (6, 1, 96, 96, 48, 30.0, [70, 1, 1, 2], [3, 300, 0, 15]),
+    (4, 4, 16, 40, 0, 0.0, [5, 1, 130], [0, 37, 6]),
+    (2, 2, 128, 128, 16, 8.0, [64, 1, 65], [10, 200, 0]),
+    (3, 3, 10, 6, 1, 2.0, [6, 2], [0, 9]),
+    (8, 2, 32, 80, 16, 12.0, [1, 1, 1], [0, 31, 200]),
+])
+def test_sigmoid_weight_attention_with_rotated_values(dt, H, G, D, Dv, half,
+                                                      cap, lens, starts):
+    """Writer: per-head unit norm after the rotation, values rotated by
+    their positions.  Attention: capped scores, per-head bias, sigmoid
+    weights without normalisation, head sums turned back; one wave per row
+    and the matrix-core kernel."""
+    page = 4
+    cache, ptab, pos, sot, slot = _paged(lens, starts, page, G * (D + Dv), dt)
+    # every cached position of every sequence gets a proper row first
+    all_lens = [s + n for s, n in zip(starts, lens)]
+    pos2 = torch.tensor([p for n in all_lens for p in range(n)],
+                        dtype=torch.int32)
+    slot2 = torch.tensor([int(ptab[b, p // page]) * page + p % page
+                          for b, n in enumerate(all_lens) for p in range(n)],
+                         dtype=torch.int32)
+    N2 = sum(all_lens)
+    inv = torch.rand(half) if half else None
+    vinv = seq.rope_inv_freq(Dv, 50.0, "cpu")
+    kv = rnd(N2, G * D + G * Dv + H * D, dt=dt)
+    c0, c1 = cache.clone(), cache.clone().to(DEV)
+    g = lambda t: None if t is None else t.to(DEV)
+    a, b = G * D, G * D + G * Dv
+    q0 = R.gqa_prepare_store(kv[:, b:], kv[:, :a], kv[:, a:b], None, None,
+                             1e-5, inv, 1.0, pos2, c0, slot2, H, G, D, Dv,
+                             True, vinv)
+    kd = kv.to(DEV)
+    q1 = seq.gqa_prepare_store(kd[:, b:], kd[:, :a], kd[:, a:b], None, None,
+                               1e-5, g(inv), 1.0, g(pos2), c1, g(slot2), H, G,
+                               D, Dv, True, g(vinv))
+    torch.testing.assert_close(q1.cpu().float(), q0.float(), **tol(dt))
+    torch.testing.assert_close(c1.cpu().float(), c0.float(), **tol(dt))
+    # the queries of this step's rows
+    rows = torch.cat([torch.arange(s, s + n) + sum(all_lens[:i])
+                      for i, (s, n) in enumerate(zip(starts, lens))])
+    q = q0[rows].contiguous()
+    pb = rnd(H) - 2.0
+    gfull = rnd(len(rows), H + 3, dt=dt)
+    scale = 4.0 / math.sqrt(D)
+    for gate in (None, gfull[:, 1:1 + H]):
+        want = R.gqa_window_attention(
+            q, c0, ptab, sot, pos, H, G, D, Dv, 1 << 30, 0, None, None, gate,
+            scale, dt, softcap=cap, head_bias=pb, sigmoid_weights=True,
+            v_inv_freq=vinv)
+        for tl in (None, seq.attention_tiles(lens, DEV)):
+            got = seq.gqa_window_attention(
+                g(q), g(c0), g(ptab), g(sot), g(pos), H, G, D, Dv, 1 << 30, 0,
+                None, None,
+                None if gate is None else gfull.to(DEV)[:, 1:1 + H], scale,
+                dt, tiles=tl, softcap=cap, head_bias=g(pb),
+                sigmoid_weights=True, v_inv_freq=g(vinv))
+            ref = want.float()
+            lim = dict(rtol=2e-2, atol=2e-2 * float(ref.abs().max())) \
+                if dt == torch.bfloat16 else dict(rtol=1e-4, atol=1e-4)
+            torch.testing.assert_close(got.cpu().float(), ref, **lim)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_head_gate_and_causal_latent_attention_without_sink(dt):
+    N, H, Dv = 11, 5, 12
+    big, gate = rnd(N, H * Dv + 4, dt=dt), rnd(N, H + 2, dt=dt)
+    want = R.sigmoid_mul_heads(big[:, 2:2 + H * Dv], gate[:, 1:1 + H])
+    got = seq.sigmoid_mul_heads(big.to(DEV)[:, 2:2 + H * Dv],
+                                gate.to(DEV)[:, 1:1 + H])
+    torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dt))
+    lens, starts, page = [70, 1, 3], [5, 300, 0], 4
+    R_, rd, H = 32, 8, 4
+    cache, ptab, pos, sot, slot = _paged(lens, starts, page, R_ + rd, dt)
+    ql, qr = rnd(sum(lens), H, R_, dt=dt), rnd(sum(lens), H, rd, dt=dt)
+    want = R.latent_window_attention(ql, qr, cache, ptab, sot, pos, 1 << 30,
+                                     None, 0.3, dt)
+    g = lambda t: t.to(DEV)
+    for tl in (None, seq.attention_tiles(lens, DEV)):
+        got = seq.latent_window_attention(g(ql), g(qr), g(cache), g(ptab),
+                                          g(sot), g(pos), 1 << 30, None, 0.3,
+                                          dt, tiles=tl)
+        torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dt))
+
+
+@pytest.mark.parametrize("N,top,E", [(1, 2, 4), (37, 3, 5), (200, 4, 8)])
+def test_gated_routed_experts_bf16(N, top, E):
+    dt = torch.bfloat16
+    Wd, ff = 96, 64
+    h = rnd(N, Wd, dt=dt)
+    idx = torch.stack([torch.randperm(E)[:top] for _ in range(N)]).int()
+    w = torch.rand(N, top)
+    gu, down = rnd(E, 2 * ff, Wd, dt=dt, scale=0.1), \
+        rnd(E, Wd, ff, dt=dt, scale=0.1)
+    ys0 = R.moe_routed_ffn(h, idx, gu, down, True)
+    assert seq.moe_routed_ffn_supported(h.to(DEV), top, ff)
+    ys1 = seq.moe_routed_ffn(h.to(DEV), idx.to(DEV), gu.to(DEV), down.to(DEV),
+                             True)
+    torch.testing.assert_close(ys1.cpu().float(), ys0.float(), **tol(dt))
+    want = R.moe_weighted_combine(ys0, idx, w, h, None, E, 1e-20, dt, 1.5)
+    got = seq.moe_weighted_combine(ys1, idx.to(DEV), w.to(DEV), h.to(DEV),
+                                   None, E, 1e-20, dt, 1.5)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dt))
