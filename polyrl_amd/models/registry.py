@@ -114,16 +114,18 @@ def _hybrid_presets():
         "nasipel-debug": lambda: nasipel_preset(
             width=64, layers=4, vocab=300, heads=4, kv_heads=2, experts=6,
             top=2, expert_ff=32),
-        # bench pairs: beside llama-400m / llama3-1b / llama3-8b-l8
+        # bench pairs: beside kuforax-400m / -1b / -8b-l8 (equal width,
+        # depth, heads, vocabulary and expert count; the gated experts'
+        # hidden size is set so that the parameter totals agree within 2 %)
         "nasipel-400m": lambda: nasipel_preset(
             width=1024, layers=12, vocab=32000, heads=16, kv_heads=4,
-            experts=8, top=2, expert_ff=2048),
+            experts=8, top=2, expert_ff=1472),
         "nasipel-1b": lambda: nasipel_preset(
             width=2048, layers=16, vocab=128256, heads=32, kv_heads=8,
-            experts=16, top=2, expert_ff=2560),
+            experts=16, top=2, expert_ff=1728),
         "nasipel-8b-l8": lambda: nasipel_preset(
             width=4096, layers=8, vocab=128256, heads=32, kv_heads=8,
-            experts=16, top=2, expert_ff=3584),
+            experts=16, top=2, expert_ff=2496),
         # tiny looped stack for CPU unit tests / fast GPU smoke
         "vurivik-debug": lambda: vurivik_preset(
             width=64, layers=4, vocab=300, heads=4, kv_heads=2, ff_mult=2.5,

@@ -97,7 +97,7 @@ __global__ __launch_bounds__(256) void gqa_prepare_kernel(
 }
 
 // One wave per head of a token (H query heads, G key heads, G value heads;
-// four waves a block take them in turn).  Query / key heads: rotate the
+// four heads a block, grid (tokens, heads / 4)).  Query / key heads: rotate the
 // first 2*half entries, then (unit) divide the head by its root mean square;
 // the statistics are taken of the rotated numbers, which are computed again
 // for the store (nothing is rounded in between).  Value heads: rotate all Dv
@@ -114,7 +114,9 @@ __global__ __launch_bounds__(256) void gqa_prepare_heads_kernel(
   const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const float pos = (float)positions[n];
   T* crow = cache + (long)slot_mapping[n] * (G * (D + Dv));
-  for (int hu = wid; hu < H + 2 * G; hu += 4) {
+  {
+    const int hu = blockIdx.y * 4 + wid;
+    if (hu >= H + 2 * G) return;          // whole wave; no barrier follows
     const T* src;
     T* dst;
     int dim, hf;
@@ -211,7 +213,7 @@ void seq_gqa_prepare_store(torch::Tensor q_out, torch::Tensor q,
       TORCH_CHECK(Dv % 2 == 0 && v_inv_freq.numel() == Dv / 2,
                   "one frequency per value pair");
     }
-    SEQ_DISPATCH_T(ty, { hipLaunchKernelGGL((gqa_prepare_heads_kernel<T>), dim3(N), dim3(256), 0, stream,
+    SEQ_DISPATCH_T(ty, { hipLaunchKernelGGL((gqa_prepare_heads_kernel<T>), dim3(N, (H + 2 * G + 3) / 4), dim3(256), 0, stream,
         (T*)q_out.data_ptr(), (const T*)q.data_ptr(), q.stride(0),
         (const T*)k.data_ptr(), k.stride(0), (const T*)v.data_ptr(),
         v.stride(0), (float)eps,

@@ -622,9 +622,10 @@ void seq_moe_combine(torch::Tensor res, torch::Tensor y, torch::Tensor inv,
 // the new row, (x - mean) * rsqrt(var + eps), is written once per weight
 // vector: out1 = unit * w1, out2 = unit * w2.  Two sublayers that read the
 // same stream share the statistics, so their norms cost one pass.  The
-// variance is the mean of the squared deviations (second pass over values
-// the thread itself wrote).
-template <typename T>
+// variance is the mean of the squared deviations.  A row of up to 256*EPT
+// numbers stays in registers between the passes (EPT > 0); longer rows
+// (EPT = 0) are read again from the values the thread itself wrote.
+template <typename T, int EPT>
 __global__ __launch_bounds__(256) void gated_add_layernorm_kernel(
     T* __restrict__ out1, T* __restrict__ out2, float* __restrict__ res,
     const T* __restrict__ y1, long ld1, const T* __restrict__ g1, long ldg1,
@@ -634,8 +635,7 @@ __global__ __launch_bounds__(256) void gated_add_layernorm_kernel(
   __shared__ float red[8], red2[8];
   const long row = blockIdx.x;
   float* rr = res + row * D;
-  float sum = 0.f;
-  for (int i = threadIdx.x; i < D; i += 256) {
+  auto joined = [&](int i) {
     float f = rr[i];
     if (y1) {
       float a = ldf(y1 + row * ld1 + i);
@@ -648,8 +648,38 @@ __global__ __launch_bounds__(256) void gated_add_layernorm_kernel(
       f += a;
       rr[i] = f;
     }
-    sum += f;
+    return f;
+  };
+  float sum = 0.f;
+  if (EPT > 0) {
+    float v[EPT > 0 ? EPT : 1];
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) {
+      const int i = threadIdx.x + e * 256;
+      v[e] = i < D ? joined(i) : 0.f;
+      sum += v[e];
+    }
+    if (!out1) return;
+    const float mean = block_reduce_sum<4>(sum, red) / D;
+    float sq = 0.f;
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) {
+      const float d = v[e] - mean;
+      if (threadIdx.x + e * 256 < D) sq += d * d;
+    }
+    const float inv = rsqrtf(block_reduce_sum<4>(sq, red2) / D + eps);
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) {
+      const int i = threadIdx.x + e * 256;
+      if (i < D) {
+        const float u = (v[e] - mean) * inv;
+        stf(out1 + row * D + i, u * w1[i]);
+        if (out2) stf(out2 + row * D + i, u * w2[i]);
+      }
+    }
+    return;
   }
+  for (int i = threadIdx.x; i < D; i += 256) sum += joined(i);
   if (!out1) return;
   const float mean = block_reduce_sum<4>(sum, red) / D;
   float sq = 0.f;
@@ -664,6 +694,14 @@ __global__ __launch_bounds__(256) void gated_add_layernorm_kernel(
     if (out2) stf(out2 + row * D + i, u * w2[i]);
   }
 }
+
+#define GALN_LAUNCH(EPTV)                                                     \
+  hipLaunchKernelGGL((gated_add_layernorm_kernel<T, EPTV>), dim3(rows),     \
+        dim3(256), 0, stream, h1 ? (T*)out1.data_ptr() : nullptr,             \
+        h2 ? (T*)out2.data_ptr() : nullptr, res.data_ptr<float>(), p(y1),     \
+        ld(y1), p(g1), ld(g1), p(y2), ld(y2), p(g2), ld(g2),                  \
+        h1 ? w1.data_ptr<float>() : nullptr,                                  \
+        h2 ? w2.data_ptr<float>() : nullptr, D, (float)eps)
 
 void seq_gated_add_layernorm(torch::Tensor out1, torch::Tensor out2,
                              torch::Tensor res, torch::Tensor y1,
@@ -700,12 +738,10 @@ void seq_gated_add_layernorm(torch::Tensor out1, torch::Tensor out2,
     auto p = [&](const torch::Tensor& t) {
       return has(t) ? (const T*)t.data_ptr() : (const T*)nullptr; };
     auto ld = [&](const torch::Tensor& t) { return has(t) ? t.stride(0) : 0L; };
-    hipLaunchKernelGGL((gated_add_layernorm_kernel<T>), dim3(rows), dim3(256),
-        0, stream, h1 ? (T*)out1.data_ptr() : nullptr,
-        h2 ? (T*)out2.data_ptr() : nullptr, res.data_ptr<float>(), p(y1),
-        ld(y1), p(g1), ld(g1), p(y2), ld(y2), p(g2), ld(g2),
-        h1 ? w1.data_ptr<float>() : nullptr,
-        h2 ? w2.data_ptr<float>() : nullptr, D, (float)eps);
+    if (D <= 1024) GALN_LAUNCH(4);
+    else if (D <= 2048) GALN_LAUNCH(8);
+    else if (D <= 4096) GALN_LAUNCH(16);
+    else GALN_LAUNCH(0);
   });
   HIP_CHECK_KERNEL();
 }

@@ -476,7 +476,8 @@ class Engine:
         # the host replay one captured hipGraph per batch size instead of
         # issuing every launch from Python
         self.enable_hybrid_graphs = (
-            str(dev) != "cpu" and getattr(self.model, "prenorm", False)
+            str(dev) != "cpu" and (getattr(self.model, "prenorm", False)
+                                   or getattr(self.model, "parallel", False))
             and bool(int(__import__("os").environ.get(
                 "POLYRL_HIP_GRAPHS", "1"))))
         self._graph_seen: Dict[int, int] = {}
@@ -849,7 +850,8 @@ class Engine:
             page_table=torch.from_numpy(ptab).to(dev),
             attn_tiles=ops.seq.attention_tiles(
                 [len(it[2]) for it in items], dev),
-            max_q=max((len(it[2]) for it in items), default=0)), cu
+            max_q=max((len(it[2]) for it in items), default=0),
+            ctx_lens=[it[1] + len(it[2]) for it in items]), cu
 
     def _run_mixed(self, prefill_reqs, prefill_lens, decode_reqs):
         """One forward over prompt portions and single decode tokens
@@ -893,7 +895,8 @@ class Engine:
     def _graph_wanted(self, B: int) -> bool:
         """Capture a batch size once it has recurred (a size seen only in
         passing, while requests finish one by one, stays eager)."""
-        if not self.enable_hybrid_graphs:
+        if not self.enable_hybrid_graphs or \
+                not self.model.graph_safe_decode(B):
             return False
         if B in self._graphs:
             return True

@@ -41,6 +41,8 @@ class HybridBatch:
     page_table: torch.Tensor      # (B, max_pages)
     attn_tiles: Optional[tuple] = None   # ops.seq.attention_tiles(lens)
     max_q: int = 0                # rows of the longest portion (0 = unknown)
+    ctx_lens: Optional[List[int]] = None   # tokens each sequence holds after
+    #                                        this step (host; None = unknown)
 
 
 _TUNED = False
@@ -68,7 +70,31 @@ def _mm(x: torch.Tensor, w: torch.Tensor,
 
 
 class _Part:
-    """Buffers of one mixer / feed-forward with their checkpoint names."""
+    """Buffers of one mixer / feed-forward with their checkpoint names.
+
+    A mixer with ``TAIL`` set can carry ``tail`` further rows (with biases)
+    at the end of its fused input projection for a product that reads the
+    same input (a layer's residual gate): the rows are ``tail_w`` /
+    ``tail_b`` and every forward leaves their result in ``tail_out``."""
+    TAIL = False
+    tail_w = tail_b = tail_out = None
+
+    def _with_tail(self, rows: int, tail: int, width, device, dtype,
+                   bias: bool):
+        """(w_in, b_in) of ``rows`` own rows plus ``tail`` shared ones; the
+        bias exists when asked for or when there is a tail (zero on rows
+        that have none)."""
+        w = torch.empty(rows + tail, width, device=device, dtype=dtype)
+        b = torch.zeros(rows + tail, device=device, dtype=dtype) \
+            if bias or tail else None
+        self._rows, self._tail = rows, tail
+        if tail:
+            self.tail_w, self.tail_b = w[rows:], b[rows:]
+        return w, b
+
+    def _split_tail(self, proj):
+        if self._tail:
+            self.tail_out = proj.narrow(1, self._rows, self._tail)
 
     def named(self, prefix: str) -> Dict[str, torch.Tensor]:
         raise NotImplementedError
@@ -170,14 +196,16 @@ class RGLRUMixer(_Part):
     product with the GELU branch.  State per sequence: the recurrence's
     vector (fp32) and the convolution's last taps-1 inputs."""
 
-    def __init__(self, spec, width, device, dtype):
+    TAIL = True
+
+    def __init__(self, spec, width, device, dtype, tail=0):
         self.spec = s = spec
         C, B = s.width, s.blocks
         self.bw = bw = C // B
         z = lambda *a, dt=dtype: torch.empty(*a, device=device, dtype=dt)
         f32 = torch.float32
-        self.w_in = z(2 * C, width)
-        self.b_in = z(2 * C)
+        self.w_in, self.b_in = self._with_tail(2 * C, tail, width, device,
+                                               dtype, True)
         self.conv = z(C, s.conv, dt=f32)
         self.conv_b = z(C, dt=f32)
         self.w_gate = z(B, 2 * bw, bw, dt=f32)
@@ -187,8 +215,8 @@ class RGLRUMixer(_Part):
 
     def named(self, p):
         C, bw = self.spec.width, self.bw
-        return {p + "y": self.w_in[:C], p + "x": self.w_in[C:],
-                p + "y.b": self.b_in[:C], p + "x.b": self.b_in[C:],
+        return {p + "y": self.w_in[:C], p + "x": self.w_in[C:2 * C],
+                p + "y.b": self.b_in[:C], p + "x.b": self.b_in[C:2 * C],
                 p + "conv": self.conv, p + "conv.b": self.conv_b,
                 p + "ra": self.w_gate[:, :bw], p + "ri": self.w_gate[:, bw:],
                 p + "ra.b": self.b_gate[:, :bw],
@@ -206,6 +234,7 @@ class RGLRUMixer(_Part):
         s = self.spec
         C, B, bw, N = s.width, s.blocks, self.bw, h.shape[0]
         proj = _mm(h, self.w_in, self.b_in)
+        self._split_tail(proj)
         u = seq.causal_conv_state(proj.narrow(1, C, C), self.conv,
                                   self.conv_b,
                                   model._state(states, (li, "conv"), C),
@@ -267,7 +296,9 @@ class SSMMixer(_Part):
 
 
 class LatentAttnMixer(_Part):
-    def __init__(self, spec, width, device, dtype):
+    TAIL = True
+
+    def __init__(self, spec, width, device, dtype, tail=0):
         self.spec = s = spec
         z = lambda *a, dt=dtype: torch.empty(*a, device=device, dtype=dt)
         f32 = torch.float32
@@ -279,8 +310,9 @@ class LatentAttnMixer(_Part):
         # the output gate (per entry or per head) and (if owned) the latent
         self.n0 = s.q_rank if s.q_rank > 0 else self.nq
         self.ng = self.nv if s.gate == "element" else s.heads
-        self.w_in = z(self.n0 + self.ng + (self.row if self.owner else 0),
-                      width)
+        self.w_in, self.b_in = self._with_tail(
+            self.n0 + self.ng + (self.row if self.owner else 0), tail, width,
+            device, dtype, False)
         self.dq_norm = z(s.q_rank, dt=f32) if s.q_rank > 0 else None
         self.uq = z(self.nq, s.q_rank) if s.q_rank > 0 else None
         self.dkv_norm = z(s.kv_rank, dt=f32) if self.owner else None
@@ -310,14 +342,15 @@ class LatentAttnMixer(_Part):
         if self.sink is not None:
             out[p + "sink"] = self.sink
         if self.owner:
-            out[p + "dkv"] = self.w_in[b:]
+            out[p + "dkv"] = self.w_in[b:b + self.row]
             out[p + "dkv.norm"] = self.dkv_norm
         return out
 
     def forward(self, h, bt, li, model, cache, states):
         s = self.spec
         N, H = h.shape[0], s.heads
-        proj = _mm(h, self.w_in)
+        proj = _mm(h, self.w_in, self.b_in)
+        self._split_tail(proj)
         rows = cache.rows[li if self.owner else s.kv_from]
         if self.owner:
             seq.latent_kv_store(proj.narrow(1, self.n0 + self.ng, self.row),
@@ -334,6 +367,8 @@ class LatentAttnMixer(_Part):
         q = q.unflatten(1, (H, s.dim + s.rot_dim))
         seq.rope_partial_(q, s.dim, self.inv_freq, bt.positions, self.amp,
                           self.interleaved)
+        if self._expand_pays(h, bt, q):
+            return _mm(self._attend_expanded(q, proj, rows, bt), self.wo)
         # absorb the key up-projection into the query: (q . W_uk c) =
         # (W_uk^T q) . c, so every head scores against the cached latent
         q_lat = torch.bmm(q[:, :, :s.dim].transpose(0, 1),
@@ -351,14 +386,69 @@ class LatentAttnMixer(_Part):
             seq.sigmoid_mul_heads(o, gate)
         return _mm(o, self.wo)
 
+    def _expand_pays(self, h, bt, q) -> bool:
+        """Steps that hold a prompt portion attend in the expanded form when
+        the matrix-core grouped-query kernel serves the head sizes and the
+        sequences' contexts are not much larger than the step itself: scoring
+        against per-head keys of dim + rot_dim numbers costs a fraction of
+        scoring every head against the whole latent row."""
+        s = self.spec
+        return (bt.ctx_lens is not None and h.is_cuda
+                and bt.attn_tiles is not None and bt.attn_tiles[2] == 0
+                and seq.gqa_mfma_supported(q, s.dim + s.rot_dim, s.vdim)
+                and sum(bt.ctx_lens) <= max(4 * h.shape[0], 4096))
+
+
+    def _attend_expanded(self, q, proj, rows, bt):
+        """Keys [W_uk c | shared rotated part] and values W_uv c of every cached
+        row the step can see, written as temporary K/V rows (one page run per
+        sequence), then grouped-query attention with one key/value head per
+        query head.  Returns the gated head outputs (N, H*Dv)."""
+        s = self.spec
+        H, D, Dr, Dv, R = s.heads, s.dim, s.rot_dim, s.vdim, s.kv_rank
+        N, dev = q.shape[0], q.device
+        ps = rows.shape[1]
+        lens = np.asarray(bt.ctx_lens, dtype=np.int64)
+        pages = -(-lens // ps)
+        base = np.concatenate([[0], np.cumsum(pages)[:-1]])       # first page
+        seq_i = np.repeat(np.arange(len(lens)), lens)
+        pos = np.concatenate([np.arange(n) for n in lens]) if len(lens) else \
+            np.zeros(0, dtype=np.int64)
+        seq_d = torch.from_numpy(seq_i).to(dev)
+        pos_d = torch.from_numpy(pos).to(dev)
+        src = bt.page_table[seq_d, pos_d // ps].long() * ps + pos_d % ps
+        dst = torch.from_numpy(base[seq_i] * ps + pos).to(dev)
+        lat = rows.view(-1, rows.shape[-1])[src]                   # (T, R + Dr)
+        c = lat[:, :R]
+        nk = H * (D + Dr)
+        tmp = torch.empty(int(pages.sum()) * ps, nk + H * Dv, device=dev,
+                          dtype=q.dtype)
+        keys = torch.empty(c.shape[0], H, D + Dr, device=dev, dtype=q.dtype)
+        keys[:, :, :D] = _mm(c, self.uk).view(-1, H, D)
+        keys[:, :, D:] = lat[:, R:].unsqueeze(1)
+        tmp[dst, :nk] = keys.view(-1, nk)
+        tmp[dst, nk:] = _mm(c, self.uv)
+        ptab = torch.from_numpy(
+            (base[:, None] + np.arange(max(int(pages.max()), 1))[None, :])
+            .astype(np.int32)).to(dev)
+        gate = proj.narrow(1, self.n0, self.ng)
+        o = seq.gqa_window_attention(
+            q.reshape(N, nk).contiguous(), tmp.view(-1, ps, nk + H * Dv), ptab,
+        bt.seq_of_tok,
+            bt.positions, H, H, D + Dr, Dv, s.window, 0, None, None,
+            gate if s.gate == "head" else None, s.scale, q.dtype,
+            tiles=bt.attn_tiles, sink=self.sink)
+        return o if s.gate == "head" else seq.sigmoid_mul(o, gate)
+
 
 class WindowAttnMixer(_Part):
     """Grouped-query attention over a sliding window of paged K/V rows
     (models.hybrid.WindowAttnSpec): one fused projection for queries, keys,
     values (unless the keys serve as values) and the per-head gate; one
     kernel norms, rotates and writes the cache rows; one attends."""
+    TAIL = True
 
-    def __init__(self, spec, width, device, dtype):
+    def __init__(self, spec, width, device, dtype, tail=0):
         self.spec = s = spec
         z = lambda *a, dt=dtype: torch.empty(*a, device=device, dtype=dt)
         f32 = torch.float32
@@ -366,11 +456,10 @@ class WindowAttnMixer(_Part):
         self.nv = 0 if s.values_from_keys else s.kv_heads * s.vdim
         self.ng = s.heads if s.head_gate else 0
         self.row = s.kv_heads * (s.dim + s.vdim)
-        self.w_in = z(self.nq + self.nk + self.nv + self.ng, width)
-        self.b_in = z(self.nq + self.nk + self.nv + self.ng) \
-            if s.qkv_bias else None
-        if self.b_in is not None:
-            self.b_in.zero_()             # the head gate has no bias
+        # (the head gate has no bias: its entries stay zero)
+        self.w_in, self.b_in = self._with_tail(
+            self.nq + self.nk + self.nv + self.ng, tail, width, device, dtype,
+            s.qkv_bias)
         self.sink = z(s.heads, dt=f32) if s.sink else None
         self.head_bias = z(s.heads, dt=f32) if s.head_bias else None
         self.v_inv_freq = seq.rope_inv_freq(s.vdim, s.value_rope_base,
@@ -392,18 +481,19 @@ class WindowAttnMixer(_Part):
 
     def named(self, p):
         a, b = self.nq, self.nq + self.nk
+        s_bias = self.spec.qkv_bias
         out = {p + "q": self.w_in[:a], p + "k": self.w_in[a:b],
                p + "o": self.wo}
         if self.nv:
             out[p + "v"] = self.w_in[b:b + self.nv]
         if self.ng:
-            out[p + "g"] = self.w_in[b + self.nv:]
+            out[p + "g"] = self.w_in[b + self.nv:b + self.nv + self.ng]
         if self.q_norm is not None:
             out[p + "q.norm"] = self.q_norm
             out[p + "k.norm"] = self.k_norm
         if self.rel is not None:
             out[p + "rel"] = self.rel
-        if self.b_in is not None:
+        if s_bias:
             out[p + "q.b"] = self.b_in[:a]
             out[p + "k.b"] = self.b_in[a:b]
             if self.nv:
@@ -418,6 +508,7 @@ class WindowAttnMixer(_Part):
         s = self.spec
         a, b = self.nq, self.nq + self.nk
         proj = _mm(h, self.w_in, self.b_in)
+        self._split_tail(proj)
         rows = cache.rows[li]
         q = seq.gqa_prepare_store(
             proj.narrow(1, 0, a), proj.narrow(1, a, self.nk),
@@ -738,13 +829,19 @@ class ParallelLayer:
         f32 = torch.float32
         z = lambda *a, dt=dtype: torch.empty(*a, device=device, dtype=dt)
         self.norm1 = z(W, dt=f32)
-        self.mixer = _MIXERS[L.mixer.kind](L.mixer, W, device, dtype)
+        cls = _MIXERS[L.mixer.kind]
+        # the mixer's gate reads the mixer's input: its rows ride at the end
+        # of the mixer's fused input projection where the mixer allows it
+        self.fused_gate = cfg.gated_residual and cls.TAIL
+        self.mixer = cls(L.mixer, W, device, dtype, tail=W) \
+            if self.fused_gate else cls(L.mixer, W, device, dtype)
         self.ff = None if L.ff is None else \
             _FFS[L.ff.kind](L.ff, W, cfg.vocab_size, device, dtype)
         self.norm2 = z(W, dt=f32) if self.ff is not None else None
         self.rg1 = self.rg1_b = self.rg2 = self.rg2_b = None
         if cfg.gated_residual:
-            self.rg1, self.rg1_b = z(W, W), z(W)
+            self.rg1, self.rg1_b = (self.mixer.tail_w, self.mixer.tail_b) \
+                if self.fused_gate else (z(W, W), z(W))
             if self.ff is not None:
                 self.rg2, self.rg2_b = z(W, W), z(W)
 
@@ -844,6 +941,27 @@ class HybridInferenceModel:
                 if shp is not None:
                     L.mixer.bias_rows = int(shp[0])
         return cfg
+
+    def graph_safe_decode(self, B: int) -> bool:
+        """Whether a decode step of B single tokens runs without a decision
+        on the host (so it can be captured in a graph): pre-norm stacks
+        always; parallel stacks when every routed feed-forward takes the
+        fused expert kernels (bf16, sizes in multiples of 32, a batch the
+        kernels' slot list holds)."""
+        if self.prenorm:
+            return True
+        if not self.parallel:
+            return False
+        for L in self.layers:
+            f = L.ff
+            if f is None:
+                continue
+            if not isinstance(f, RoutedMoE) or f.E == 0 or \
+                    self.dtype != torch.bfloat16 or B > 256 or \
+                    B * f.top > 1024 or self.cfg.hidden_size % 32 or \
+                    f.ff % 32:
+                return False
+        return True
 
     def cache_row_dims(self) -> Dict[int, int]:
         """Cache row size per layer RUN that owns paged rows (a looped
@@ -1140,7 +1258,8 @@ class HybridInferenceModel:
             L = self.layers[li]
             h1, h2 = self._norms(res, y1, g1, y2, g2, L.norm1, L.norm2)
             y1 = L.mixer.forward(h1, bt, ri, self, cache, states)
-            g1 = _mm(h1, L.rg1, L.rg1_b) if L.rg1 is not None else None
+            g1 = L.mixer.tail_out if L.fused_gate else \
+                _mm(h1, L.rg1, L.rg1_b) if L.rg1 is not None else None
             y2 = g2 = None
             if L.ff is not None:
                 y2 = L.ff.forward(h2, res, bt)

@@ -109,6 +109,12 @@ def run(e, rid, t, want=None, end=True):
     ("shared-cache", [(attn(window=5), None), (attn(window=9, kv_from=0,
                                                      heads=2, dim=16,
                                                      vdim=12), None)]),
+    # key (dim + rot) and value sizes in multiples of 8: bf16 prompt steps
+    # attend in the expanded form on the matrix cores
+    ("attention-expanded", [(attn(vdim=24), None)]),
+    ("shared-cache-expanded", [(attn(window=5, vdim=16), None),
+                               (attn(window=9, kv_from=0, heads=2, dim=16,
+                                     vdim=8), None)]),
     ("dense", [(DELTA, DENSE)]),
     ("experts", [(DELTA, MOE)]),
     ("one-expert", [(SSM, MOE1)]),
@@ -221,12 +227,13 @@ def test_pages_and_slots_are_reused_clean(target):
 
 
 # -------------------------------------------- windows, pages, far tokens
-def _loud_key_model(window, page_note=""):
+def _loud_key_model(window, vdim=20):
     """One attention layer (plus a sharer) where one token id has a huge
     rotated-key part, so whichever query still sees it attends to it: a
     window that is one token off changes the logits at its edge."""
-    cfg = config([(attn(window=window, rank=24), None),
-                  (attn(window=window + 3, kv_from=0, rank=24), DENSE)],
+    cfg = config([(attn(window=window, rank=24, vdim=vdim), None),
+                  (attn(window=window + 3, kv_from=0, rank=24, vdim=vdim),
+                   DENSE)],
                  taps=1, side=6)
     W = O.random_weights(cfg, seed=23)
     W["embed"][5] *= 12.0                   # token 5 = the loud key
@@ -235,9 +242,10 @@ def _loud_key_model(window, page_note=""):
 
 
 @pytest.mark.parametrize("target", TARGETS)
-@pytest.mark.parametrize("window", [4, 9, 16])
-def test_window_edge_in_prompt_and_decode(target, window):
-    cfg, W = _loud_key_model(window)
+@pytest.mark.parametrize("window,vdim", [(4, 20), (9, 20), (16, 20),
+                                         (4, 24), (9, 24), (16, 24)])
+def test_window_edge_in_prompt_and_decode(target, window, vdim):
+    cfg, W = _loud_key_model(window, vdim)
     t = [x if x != 5 else 6 for x in toks(3 * window + 9, seed=9)]
     loud = window + 1                       # crosses a page edge for page=4
     t[loud] = 5

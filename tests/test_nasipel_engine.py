@@ -360,13 +360,16 @@ def _loud_attention(width=32):
     return cfg, W
 
 
-def _loud_latent(width=32):
+def _loud_latent(width=32, dim=8):
     """The same for latent attention: the query latent's first entry reads
     the constant channel, the key/value latent's first entry reads LOUD's
     channel; every head's last unrotated query (key) entry reads that
-    latent entry, so LOUD's score towers over the others in the softmax."""
-    layer = mla(heads=3, dim=8, rot_dim=6, vdim=10, kv_rank=12, q_rank=14,
-                scale=1.0)
+    latent entry, so LOUD's score towers over the others in the softmax.
+    With dim = 10 the key size (dim + rot_dim = 16) and the value size suit
+    the matrix-core kernel, so bf16 prompt portions attend in the expanded
+    form; with dim = 8 every step scores against the latent rows."""
+    layer = mla(heads=3, dim=dim, rot_dim=6, vdim=8 if dim == 10 else 10,
+                kv_rank=12, q_rank=14, scale=1.0)
     cfg = config([(layer, None)], width=width)
     W = O.random_weights(cfg, seed=29)
     W["embed"][:, 0] = 3.0
@@ -380,22 +383,23 @@ def _loud_latent(width=32):
     W["l0.mix.dkv"][0, 1] = 4.0
     W["l0.mix.dkv.norm"][0] = 1.0
     for h in range(3):
-        W["l0.mix.uq"][h * 14 + 7] = 0.0
-        W["l0.mix.uq"][h * 14 + 7, 0] = 2.0
-        W["l0.mix.uk"][h * 8 + 7] = 0.0
-        W["l0.mix.uk"][h * 8 + 7, 0] = 2.0
+        W["l0.mix.uq"][h * (dim + 6) + dim - 1] = 0.0
+        W["l0.mix.uq"][h * (dim + 6) + dim - 1, 0] = 2.0
+        W["l0.mix.uk"][h * dim + dim - 1] = 0.0
+        W["l0.mix.uk"][h * dim + dim - 1, 0] = 2.0
     return cfg, W
 
 
 @pytest.mark.parametrize("target", TARGETS)
 @pytest.mark.parametrize("where", [0, 3, 4, 63, 64, 65])
-@pytest.mark.parametrize("kind", ["attention", "latent"])
+@pytest.mark.parametrize("kind", ["attention", "latent", "latent-expanded"])
 def test_far_key_at_page_borders(target, where, kind):
     """LOUD at the first position and on both sides of page borders (pages
     of 4 and, for the 64-token tiles of the matrix-core kernels, position
     63..65) is seen from 230 tokens away: in one prompt, decoded token by
     token, across a cut right behind it, and in portions."""
-    cfg, W = _loud_attention() if kind == "attention" else _loud_latent()
+    cfg, W = _loud_attention() if kind == "attention" else \
+        _loud_latent(dim=10 if kind == "latent-expanded" else 8)
     n = 230 if where < 10 else 300
     t = toks(n, seed=9 + where, avoid=(LOUD,))
     t[where] = LOUD
@@ -581,3 +585,41 @@ def test_registry_preset_runs_and_resumes_memory():
     assert not e.kv.rows
     e.resume_memory()
     torch.testing.assert_close(run(e, "b", t), a)
+
+
+@pytest.mark.gpu
+def test_decode_graph_replays_match_eager_steps():
+    """Pure bf16 decode steps replay a captured graph once their batch size
+    has recurred: 40 greedy tokens (eager sampling, copies and a host sync
+    between the replays) equal the run with every launch issued eagerly,
+    also after the batch shrinks to another size.  fp32 steps sort rows by
+    expert on the host and stay eager."""
+    cfg = config([(lru(width=64, blocks=2), moe(experts=4, top=2, groups=2,
+                                                keep=1, ff=32)),
+                  (mla(), moe(experts=4, top=1, groups=1, keep=1, ff=64)),
+                  (attn(), None)], width=64)
+    W = O.random_weights(cfg, seed=47)
+    prompts = [toks(n, seed=80 + n) for n in (9, 3, 14)]
+    new = (40, 17, 40)
+    outs = {}
+    for graphs in (False, True):
+        e = engine(cfg, W, ("cuda", torch.bfloat16), slots=3)
+        assert e.enable_hybrid_graphs and e.model.graph_safe_decode(3)
+        e.enable_hybrid_graphs = graphs
+        for i, (p, n) in enumerate(zip(prompts, new)):
+            e.add_request(f"g-{i}", p, SamplingParams(temperature=0.0,
+                                                      max_new_tokens=n))
+        got = {}
+        while e.has_work():
+            for o in e.step():
+                got[o.rid] = o
+        outs[graphs] = [got[f"g-{i}"] for i in range(3)]
+        assert sorted(e._graphs) == ([2, 3] if graphs else [])
+        assert e.states.free_slots == e.states.num_slots
+    for a, b in zip(outs[False], outs[True]):
+        assert a.output_ids == b.output_ids
+        torch.testing.assert_close(torch.tensor(a.output_logprobs),
+                                   torch.tensor(b.output_logprobs),
+                                   rtol=1e-5, atol=1e-5)
+    e = engine(cfg, W, ("cuda", torch.float32), slots=3)
+    assert not e.model.graph_safe_decode(3)
