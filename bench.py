@@ -132,8 +132,8 @@ def main():
                    help="instead of the PPO step: rollout-engine prefill and "
                         "decode tokens/s of a hybrid decoder beside a dense "
                         "one of equal width and depth (registry names, "
-                        "random weights), e.g. bizusun-1b:llama3-1b or "
-                        "vurivik-1b:llama3-1b")
+                        "random weights), e.g. bizusun-1b:llama3-1b, "
+                        "vurivik-1b:llama3-1b or nasipel-1b:kuforax-1b")
     p.add_argument("--engine-prefill", type=str, default="8x2048",
                    help="engine-compare prefill workload: prompts x length")
     p.add_argument("--engine-decode", type=str, default="64x128",

@@ -1278,12 +1278,10 @@ class HybridInferenceModel:
             h = seq.gated_add_layernorm(
                 res_rows.contiguous(), None, None, None, None,
                 self.final_norm, None, self.cfg.norm_eps, self.dtype)[0]
-            return _mm(h, self.lm_head).float() * self.cfg.logit_scale \
-                if self.cfg.logit_scale != 1.0 else \
-                _mm(h, self.lm_head).float()
-        h = seq.add_rmsnorm_f32res(res_rows.contiguous(), None,
-                                   self.final_norm, self.cfg.norm_eps,
-                                   self.dtype, self.cfg.norm_offset)
+        else:
+            h = seq.add_rmsnorm_f32res(res_rows.contiguous(), None,
+                                       self.final_norm, self.cfg.norm_eps,
+                                       self.dtype, self.cfg.norm_offset)
         out = _mm(h, self.lm_head).float()
         if self.cfg.logit_scale != 1.0:
             out = out * self.cfg.logit_scale
