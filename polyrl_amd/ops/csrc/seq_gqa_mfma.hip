@@ -26,7 +26,12 @@
 // with an L2 of its own, so the id is taken apart as XCD = id % 8 and, inside
 // an XCD's sequence, the H/G query heads that share a key/value head follow
 // each other for the same row tile: their K and V tiles are fetched into that
-// XCD's L2 once and hit there for the other heads of the group.
+// XCD's L2 once and hit there for the other heads of the group.  With eight
+// key/value heads or a multiple of that, every XCD takes whole key/value
+// heads and walks their row tiles in order: successive tiles of a sequence
+// read the same rows, which then stay in that one L2 (with few query heads
+// per group -- one, for keys expanded per head -- a round-robin over the
+// dies would make every die fetch every head's rows).
 #include <torch/extension.h>
 #include <ATen/hip/HIPContext.h>
 
@@ -72,7 +77,10 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(
   const int per = H / G;                 // query heads per key/value head
   const int xcd = blockIdx.x % GQA_XCDS;
   const int seq_in_xcd = blockIdx.x / GQA_XCDS;
-  const int unit = (seq_in_xcd / per) * GQA_XCDS + xcd;   // (tile, kv head)
+  // (tile, kv head) unit of this block
+  const int unit = G % GQA_XCDS == 0
+      ? xcd * (ntiles_rows * (G / GQA_XCDS)) + seq_in_xcd / per
+      : (seq_in_xcd / per) * GQA_XCDS + xcd;
   if (unit >= ntiles_rows * G) return;   // padding of the last round
   // later row tiles see more keys: they start first, the short ones fill
   // the end of the launch

@@ -352,6 +352,9 @@ def test_gqa_prepare_store(dt, H, G, D, Dv, half, norm, own_v):
     (4, 2, 64, 64, 16, 70, False, True, [100, 1, 40], [50, 300, 0]),
     (2, 1, 40, 24, 200, 0, True, False, [130, 1, 70], [170, 450, 0]),
     (4, 4, 96, 96, 40, 33, False, False, [1, 1, 1], [0, 31, 200]),
+    (16, 8, 32, 32, 50, 3, False, True, [130, 1, 70], [20, 90, 0]),
+    (8, 8, 24, 16, 1 << 30, 0, False, False, [200, 3], [0, 64]),
+    (16, 16, 16, 8, 90, 0, False, True, [65, 64, 1], [0, 1, 5]),
 ])
 def test_gqa_window_attention(dt, H, G, D, Dv, window, keep, bias, gate,
                               lens, starts):
@@ -643,6 +646,7 @@ def test_rotation_pairs_and_amplitude(dt, inter):
     (2, 2, 128, 128, 16, 8.0, [64, 1, 65], [10, 200, 0]),
     (3, 3, 10, 6, 1, 2.0, [6, 2], [0, 9]),
     (8, 2, 32, 80, 16, 12.0, [1, 1, 1], [0, 31, 200]),
+    (8, 8, 32, 32, 8, 6.0, [130, 2, 67], [0, 40, 64]),
 ])
 def test_sigmoid_weight_attention_with_rotated_values(dt, H, G, D, Dv, half,
                                                       cap, lens, starts):
