@@ -913,7 +913,7 @@ def nasipel_preset(width: int, layers: int, vocab: int = 32000,
                 heads=heads, kv_heads=kv_heads, dim=hd, vdim=hd,
                 window=UNBOUNDED, scale=1.0 / math.sqrt(hd),
                 rope=RopeSpec(dims=hd, base=10000.0), head_unit_norm=True,
-                softcap=30.0, head_bias=True, weights="sigmoid",
+                softcap=50.0, head_bias=True, weights="sigmoid",
                 value_rope_base=10000.0)
         else:
             mixer = LatentAttnSpec(
@@ -921,11 +921,11 @@ def nasipel_preset(width: int, layers: int, vocab: int = 32000,
                 kv_rank=4 * hd, window=UNBOUNDED,
                 scale=1.0 / math.sqrt(hd + hd // 2), q_rank=6 * hd,
                 sink=False, gate="head",
-                rope=RopeSpec(dims=hd // 2, base=10000.0, factor=4.0,
+                rope=RopeSpec(dims=hd // 2, base=10000.0, factor=8.0,
                               original=4096.0, interleaved=True))
         ff = FFSpec("routed_moe", expert_ff, experts, top,
                     group_count=groups, group_keep=1, router_act="sigmoid",
-                    group_top=2, route_scale=1.5, expert_act="silu_gated")
+                    group_top=2, route_scale=2.5, expert_act="silu_gated")
         out.append(HybridLayerSpec(mixer, ff))
     return HybridConfig(arch="nasipel", vocab_size=vocab, hidden_size=width,
                         layers=out, norm_eps=1e-5, canon_taps=1,

@@ -63,7 +63,7 @@ def mla(heads=3, dim=8, rot_dim=6, vdim=10, kv_rank=12, q_rank=14,
                       "scale": scale, "rot": r}}
 
 
-def moe(experts=6, top=2, groups=3, keep=2, ff=16, scale=1.5):
+def moe(experts=6, top=2, groups=3, keep=2, ff=16, scale=1.25):
     return {"kind": "moe", "expert": {"ff": ff},
             "router": {"experts": experts, "top": top, "scale": scale,
                        "groups": {"count": groups, "keep": keep}}}

@@ -740,7 +740,7 @@ def test_gated_routed_experts_bf16(N, top, E):
     ys1 = seq.moe_routed_ffn(h.to(DEV), idx.to(DEV), gu.to(DEV), down.to(DEV),
                              True)
     torch.testing.assert_close(ys1.cpu().float(), ys0.float(), **tol(dt))
-    want = R.moe_weighted_combine(ys0, idx, w, h, None, E, 1e-20, dt, 1.5)
+    want = R.moe_weighted_combine(ys0, idx, w, h, None, E, 1e-20, dt, 1.75)
     got = seq.moe_weighted_combine(ys1, idx.to(DEV), w.to(DEV), h.to(DEV),
-                                   None, E, 1e-20, dt, 1.5)
+                                   None, E, 1e-20, dt, 1.75)
     torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dt))
