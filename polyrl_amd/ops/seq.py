@@ -1,10 +1,11 @@
 """Sequence-mixer ops for hybrid decoders: fp32-residual norms (plain and
-offset weights, fused joints, scaled branches), the composed embedding
-(scaled row + hashed pair row + sinusoid), stateful causal convolutions, the
-generalised delta rule, gated linear attention, the selective state-space
-scan, windowed latent attention with a softmax sink, grouped-query (window or
-causal) attention over paged K/V rows, and table-routed or router-chosen
-expert feed-forwards.
+offset weights, fused joints, scaled branches, the gated layer-norm joint of
+parallel layers), the composed embedding (scaled row + hashed pair row +
+sinusoid), stateful causal convolutions, the generalised delta rule, gated
+linear attention, the selective state-space scan, the real-gated linear
+recurrence, windowed or causal latent attention with an optional softmax
+sink, grouped-query (window or causal; softmax or sigmoid weights) attention
+over paged K/V rows, and table-routed or router-chosen expert feed-forwards.
 
 Same policy as the rest of ``polyrl_amd.ops``: on a HIP device the in-tree
 extension is REQUIRED (csrc/seq_*.hip, templated on the activation type:
